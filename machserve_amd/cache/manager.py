@@ -2,12 +2,12 @@
 per-request state of fixed size.
 
 Layers are sorted into *groups* by what they need: all keys ("full"), or a window of the
-most recent ``W`` keys ("window{W}").  Each group has a page pool and block tables of its
+most recent ``W`` keys ("window{W}"; "window{W}+first{F}" if the request's first ``F`` tokens stay visible beside them).  Each group has a page pool and block tables of its
 own, shared by the layers of the group (one page id addresses the same page in each of
 their K and V pools, as in ``crates/mach-model/src/paged_kv.rs:3-5``).  Pages are taken when
 a step needs them, one logical page at a time, and given back when the request ends or,
-in a window group, when every later row's window has passed the page; freed pages are
-handed out again.  A request also holds one *state slot*: an index into arrays
+in a window group, when every later row's window has passed the page (the pages of first tokens
+that stay visible excepted); freed pages are handed out again.  A request also holds one *state slot*: an index into arrays
 ``[slots, ...]`` that mixers with state of fixed size own, zeroed on admission
 (the reference indexes its recurrent state by slot the same way,
 ``crates/mach-model/src/batched.rs:410-415, 2644-2683``).
@@ -27,8 +27,10 @@ from typing import Dict, List, Optional, Tuple
 from . import CacheCore, CacheError
 
 
-def group_name(window: Optional[int]) -> str:
-    return "full" if window is None else f"window{window}"
+def group_name(window: Optional[int], keep_first: int = 0) -> str:
+    if window is None:
+        return "full"
+    return f"window{window}" + (f"+first{keep_first}" if keep_first else "")
 
 
 @dataclass
@@ -38,6 +40,7 @@ class GroupSpec:
     kv_heads: int
     head_dim: int
     v_head_dim: int = 0      # width of a value; the key's width unless the request says otherwise
+    keep_first: int = 0      # a window group: the first tokens of a request that stay visible
     layers: List[Tuple[int, int]] = field(default_factory=list)  # (layer run, index among its requests)
 
 
@@ -100,7 +103,7 @@ def pages_by_need(max_tokens: int, max_requests: int, portion: int, page_size: i
     def rule(group: "GroupSpec") -> int:
         if group.window is None:
             return full
-        per_request = -(-(group.window + portion - 1) // page_size) + 1
+        per_request = -(-(group.window + portion - 1) // page_size) + 1 + -(-group.keep_first // page_size)
         return max(1, min(full, max_requests * per_request))
     return rule
 
@@ -131,14 +134,15 @@ class CacheManager:
             for j, r in enumerate(reqs):
                 if isinstance(r, PagedKVRequest):
                     v_hd = r.v_head_dim or r.head_dim
-                    name = group_name(r.window)
+                    keep = (getattr(r, "keep_first", 0) or 0) if r.window is not None else 0
+                    name = group_name(r.window, keep)
                     g = specs.get(name)
                     if g is not None and (g.kv_heads, g.head_dim, g.v_head_dim) != (r.kv_heads, r.head_dim, v_hd):
                         # same need, other geometry: a group of its own
                         name = f"{name}/kv{r.kv_heads}x{r.head_dim}" + (f"v{v_hd}" if v_hd != r.head_dim else "")
                         g = specs.get(name)
                     if g is None:
-                        g = specs[name] = GroupSpec(name, r.window, r.kv_heads, r.head_dim, v_hd)
+                        g = specs[name] = GroupSpec(name, r.window, r.kv_heads, r.head_dim, v_hd, keep_first=keep)
                     g.layers.append((i, j))
                     self.paged[(i, j)] = name
                 elif isinstance(r, SharedKVRequest):
@@ -165,7 +169,7 @@ class CacheManager:
             pages = num_pages[name] if isinstance(num_pages, dict) else num_pages(spec) if callable(num_pages) else num_pages
             if isinstance(pages, bool) or not isinstance(pages, int) or pages < 1:
                 raise CacheError(f"group {name}: {pages!r} pages; a pool needs at least one")
-            index = self.core.add_group(name, spec.window or 0, pages)
+            index = self.core.add_group(name, spec.window or 0, pages, spec.keep_first)
             self.groups[name] = _Group(spec, self.core, index)
         self._names = list(self.groups)
         self.device = None  # filled by DeviceCache

@@ -1,10 +1,12 @@
-from .specs import (AttentionSpec, ConfigError, EmbeddingSpec, GatedMlpSpec, HeadSpec, LayerSpec, ModelSpec,
-                    NormSpec, RotarySpec, YarnSpec)
+from .specs import (AttentionSpec, ConfigError, EmbeddingSpec, GatedMlpSpec, HeadSpec, LayerSpec, LightningSpec, ModelSpec,
+                    NormSpec, RotarySpec, SandwichLayerSpec, SelectiveScanSpec, TalkingAttentionSpec, YarnSpec)
 from .registry import architectures, architecture_of, config_from_dict, load_config, register_architecture
 from .qwen2 import ARCHITECTURE as QWEN2_ARCHITECTURE, Qwen2Config
+from .renanex import ARCHITECTURE as RENANEX_ARCHITECTURE, RenanexConfig
 
 register_architecture(QWEN2_ARCHITECTURE, Qwen2Config, model_type="qwen2")
+register_architecture(RENANEX_ARCHITECTURE, RenanexConfig)
 
-__all__ = ["AttentionSpec", "ConfigError", "EmbeddingSpec", "GatedMlpSpec", "HeadSpec", "LayerSpec", "ModelSpec",
-           "NormSpec", "RotarySpec", "YarnSpec", "architectures", "architecture_of", "config_from_dict", "load_config",
-           "register_architecture", "Qwen2Config", "QWEN2_ARCHITECTURE"]
+__all__ = ["AttentionSpec", "ConfigError", "EmbeddingSpec", "GatedMlpSpec", "HeadSpec", "LayerSpec", "LightningSpec", "ModelSpec",
+           "NormSpec", "RotarySpec", "SandwichLayerSpec", "SelectiveScanSpec", "TalkingAttentionSpec", "YarnSpec", "architectures", "architecture_of", "config_from_dict", "load_config",
+           "register_architecture", "Qwen2Config", "QWEN2_ARCHITECTURE", "RenanexConfig", "RENANEX_ARCHITECTURE"]

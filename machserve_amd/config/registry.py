@@ -1,4 +1,4 @@
-"""One registry from an architecture's name (``architectures[0]`` of config.json) to its
+"""One registry from an architecture's name (``architectures[0]`` or ``architecture`` of config.json) to its
 typed configuration class.  A configuration class has ``from_dict(raw) -> config``,
 ``config.to_spec() -> ModelSpec`` and, for the random-weights mode,
 ``config.random_tensor_plan()`` and ``config.to_dict()``.
@@ -32,10 +32,12 @@ def architecture_of(raw: dict) -> str:
     archs = raw.get("architectures")
     if isinstance(archs, list) and archs and isinstance(archs[0], str):
         name = archs[0]
+    elif isinstance(raw.get("architecture"), str):  # a configuration that names its one architecture
+        name = raw["architecture"]
     elif isinstance(raw.get("model_type"), str) and raw["model_type"] in _MODEL_TYPES:
         name = _MODEL_TYPES[raw["model_type"]]
     else:
-        raise ConfigError("config.json: no 'architectures' list and no known 'model_type'; "
+        raise ConfigError("config.json: no 'architectures' list, no 'architecture' and no known 'model_type'; "
                           f"supported architectures: {architectures()}")
     if name not in _ARCHITECTURES:
         raise ConfigError(f"config.json: architecture {name!r} is not supported; supported: {architectures()}")

@@ -51,6 +51,11 @@ class RotarySpec:
     theta: float
     tensors: Mapping[str, str] = field(default_factory=dict)
     yarn: Optional[YarnSpec] = None
+    # how many numbers of a head are rotated, the first ones (None: all of them); the frequencies and YaRN's pair
+    # indices are then those of a head of this size
+    rotary_dim: Optional[int] = None
+    # the precision in which the table of frequencies is worked out before it is rounded to 32-bit
+    table_precision: str = "float32"
 
 
 @dataclass(frozen=True)
@@ -76,6 +81,62 @@ class AttentionSpec:
 
 
 @dataclass(frozen=True)
+class TalkingAttentionSpec:
+    """Grouped-query attention whose heads exchange their scaled scores before the softmax
+    (``score_h = sum_g talk[h, g] score_g``), with keys ``head_dim`` and values ``v_head_dim`` wide.
+
+    ``qk_norm``: an RMS norm (``norm_eps``) over the whole query projection and one over the whole key projection,
+    before the rotation.  ``talk``: whether there is an exchange matrix.  ``window`` / ``keep_first``: a row sees the
+    last ``window`` positions up to its own (None: all) and the request's first ``keep_first``.  ``value_blend``:
+    None, ``"source"`` (the layer's own values are kept for the layers below to blend with) or ``"blend"``
+    (``v = (1 - w) v + w v_source`` with a learned number ``w``; the blended values are cached).
+    """
+    kind: str
+    hidden: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    position: Optional[RotarySpec]
+    scale: float
+    window: Optional[int] = None
+    keep_first: int = 0
+    qk_norm: bool = False
+    norm_eps: float = 1e-6
+    talk: bool = True
+    value_blend: Optional[str] = None
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class SelectiveScanSpec:
+    """A Mamba layer: input projection to ``[x | z]`` of ``inner`` channels each, a causal convolution of
+    ``conv_taps`` taps per channel with SiLU, step sizes from a ``dt_rank`` bottleneck, a scan over ``states``
+    states a channel, the gate ``silu(z)`` and an output projection."""
+    kind: str
+    hidden: int
+    inner: int
+    states: int
+    dt_rank: int
+    conv_taps: int
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class LightningSpec:
+    """Linear attention with one decay per head: ``S <- decay_h S + k v^T``, ``o = S^T q`` with SiLU on q, k and v; the
+    heads' outputs are normed together (``norm_eps``), gated by a sigmoid and projected."""
+    kind: str
+    hidden: int
+    heads: int
+    head_dim: int
+    v_head_dim: int
+    decay: Sequence[float]
+    norm_eps: float = 1e-6
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
 class GatedMlpSpec:
     """``down(act(gate(x)) * up(x))``."""
     kind: str
@@ -98,6 +159,19 @@ class LayerSpec:
 
 
 @dataclass(frozen=True)
+class SandwichLayerSpec:
+    """A block with a norm before and after each branch: ``x += post(mixer(pre(x)))``, then the same around the
+    feed-forward; ``feed_forward`` None: the layer has none (then its two norms are None too)."""
+    block: str
+    mixer: object
+    feed_forward: Optional[object]
+    mixer_norm: object
+    mixer_post_norm: object
+    feed_forward_norm: Optional[object]
+    feed_forward_post_norm: Optional[object]
+
+
+@dataclass(frozen=True)
 class EmbeddingSpec:
     """Token embedding: rows of a table, times ``scale``."""
     vocab: int
@@ -117,6 +191,7 @@ class HeadSpec:
     tensors: Mapping[str, str] = field(default_factory=dict)
     kind: str = "linear"
     scale: float = 1.0  # the logits are multiplied by it
+    softcap: float = 0.0  # then ``softcap * tanh(logits / softcap)``; 0: no cap
 
 
 @dataclass(frozen=True)

@@ -142,6 +142,34 @@ __global__ __launch_bounds__(256) void add_partials_kernel(float* __restrict__ x
     x[i] = v;
 }
 
+// x[t, :] += y / sqrt(mean(y^2) + eps) * w with y = sum_p partials[p, t, :] (in order): a branch's output, given as
+// the partial sums of its last product, normalised and added to the stream in one pass.
+__global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ x, const float* __restrict__ partials, int n_partials,
+                                                       size_t partial_stride, const float* __restrict__ w, int d, float eps) {
+    __shared__ float scratch[4];
+    extern __shared__ float vals[];  // d floats: the summed row
+    const size_t r = blockIdx.x;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < d; c += 256) {
+        float v = 0.f;
+        for (int p = 0; p < n_partials; ++p) v += partials[p * partial_stride + r * d + c];
+        vals[c] = v;
+        ss += v * v;
+    }
+    ss = block_sum<256>(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    float* dst = x + r * d;
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] += vals[c] * inv * w[c];
+}
+
+// v = logits * scale;  logits = cap > 0 ? cap * tanh(v / cap) : v
+__global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ logits, size_t n, float scale, float cap) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float v = logits[i] * scale;
+    logits[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+}
+
 struct RopeArgs {
     const float* qkv;       // [n_partials, T, stride] partial sums of: q heads, then (if written) k heads, v heads
     const float* bias;      // [stride] or null, added to the sum
@@ -370,6 +398,21 @@ extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T
         hipLaunchKernelGGL(rmsnorm_kernel<elem_t>, dim3(n), dim3(256), smem, stream, x, partials, n_partials, ps, rows, w,
                            (elem_t*)out, d, eps);
     return check_launch("rmsnorm");
+}
+
+extern "C" int ms_norm_add(float* x, const float* partials, int n_partials, const float* w, int T, int d, float eps, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && d > 0 && n_partials > 0, "norm_add: empty problem T=%d d=%d with %d sums", T, d, n_partials);
+    MS_REQUIRE(d <= MAX_ROW_FLOATS, "norm_add: width %d exceeds the row buffer of %d", d, MAX_ROW_FLOATS);
+    MS_REQUIRE(x && partials && w, "norm_add: a buffer is missing");
+    hipLaunchKernelGGL(norm_add_kernel, dim3(T), dim3(256), (size_t)d * sizeof(float), stream, x, partials, n_partials, (size_t)T * d, w,
+                       d, eps);
+    return check_launch("norm_add");
+}
+
+extern "C" int ms_softcap(float* logits, long n, float scale, float cap, hipStream_t stream) {
+    MS_REQUIRE(n > 0 && logits, "softcap: empty problem");
+    hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, logits, (size_t)n, scale, cap);
+    return check_launch("softcap");
 }
 
 extern "C" int ms_add_partials(float* x, const float* partials, int n_partials, int T, int d, hipStream_t stream) {

@@ -104,11 +104,12 @@ private:
 
 struct Group {
     std::string name;
-    int window;  // keys a row may see; 0 = all
+    int window;      // keys a row may see; 0 = all
+    int keep_first;  // with a window: a request's first tokens stay visible, so the pages that hold them are never given back
     BlockPool pool;
     std::unordered_map<int, std::vector<int>> tables;  // slot -> logical page -> physical page, -1 = given back
     std::unordered_map<int, int> first_live;           // slot -> first logical page not yet given back
-    Group(std::string n, int w, int pages) : name(std::move(n)), window(w), pool(pages) {}
+    Group(std::string n, int w, int pages, int keep) : name(std::move(n)), window(w), keep_first(keep), pool(pages) {}
 };
 
 class CacheCore {
@@ -117,8 +118,9 @@ public:
         if (page_size < 16 || page_size % 16) throw CacheError(cat("page size ", page_size, " must be a positive multiple of 16"));
         if (max_requests < 1) throw CacheError("at least one request slot is needed");
     }
-    int add_group(const std::string& name, int window, int num_pages) {
-        groups_.emplace_back(name, window, num_pages);
+    int add_group(const std::string& name, int window, int num_pages, int keep_first = 0) {
+        if (keep_first < 0) throw CacheError(cat("group ", name, ": ", keep_first, " first tokens kept"));
+        groups_.emplace_back(name, window, num_pages, window > 0 ? keep_first : 0);
         return (int)groups_.size() - 1;
     }
     int page_size() const { return page_size_; }
@@ -126,6 +128,9 @@ public:
     int num_groups() const { return (int)groups_.size(); }
     const std::string& group_name(int g) const { return groups_.at(g).name; }
     int group_window(int g) const { return groups_.at(g).window; }
+    int group_keep_first(int g) const { return groups_.at(g).keep_first; }
+    // pages at the start of a request that a window group never gives back
+    int group_kept_pages(int g) const { return (groups_.at(g).keep_first + page_size_ - 1) / page_size_; }
     int group_pages(int g) const { return groups_.at(g).pool.num_pages(); }
     int group_available(int g) const { return groups_.at(g).pool.available(); }
     std::vector<int> group_live_pages(int g) const { return groups_.at(g).pool.live_pages(); }
@@ -187,8 +192,9 @@ public:
             // the next row is at position L and sees keys > L - window
             auto& table = g.tables[slot];
             const int dead = std::min((int)table.size(), std::max(0, L - g.window + 1) / page_size_);
+            const int kept = (g.keep_first + page_size_ - 1) / page_size_;  // these hold first tokens that stay visible
             int& first = g.first_live[slot];
-            for (int p = first; p < dead; ++p)
+            for (int p = std::max(first, kept); p < dead; ++p)
                 if (table[p] >= 0) {
                     g.pool.free(table[p]);
                     table[p] = -1;

@@ -33,7 +33,9 @@ PYBIND11_MODULE(ms_host, m) {
         .def("is_live", &SlotPool::is_live);
     py::class_<CacheCore>(m, "CacheCore")
         .def(py::init<int, int>())
-        .def("add_group", &CacheCore::add_group)
+        .def("add_group", &CacheCore::add_group, py::arg("name"), py::arg("window"), py::arg("num_pages"), py::arg("keep_first") = 0)
+        .def("group_keep_first", &CacheCore::group_keep_first)
+        .def("group_kept_pages", &CacheCore::group_kept_pages)
         .def_property_readonly("page_size", &CacheCore::page_size)
         .def_property_readonly("max_requests", &CacheCore::max_requests)
         .def("num_groups", &CacheCore::num_groups)

@@ -57,7 +57,8 @@ public:
             // portion at most; a group of all keys holds every page of the request
             int pages = (total + ps - 1) / ps;
             const int window = cache_.group_window(g);
-            if (window > 0) pages = std::min(pages, (window + std::min(chunk_, budget_) - 1 + ps - 1) / ps + 1);
+            // (and the pages of the first tokens that the group keeps visible)
+            if (window > 0) pages = std::min(pages, (window + std::min(chunk_, budget_) - 1 + ps - 1) / ps + 1 + cache_.group_kept_pages(g));
             if (pages > cache_.group_pages(g))
                 throw SchedulerError(cat("request of up to ", total, " cached tokens needs ", pages, " pages at a time; group ",
                                          cache_.group_name(g), " has ", cache_.group_pages(g)));

@@ -77,6 +77,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time, each rounded up to the page size")
     ap.add_argument("--page-size", type=int, default=64)
+    ap.add_argument("--max-requests", type=int, default=4, help="requests that are live at any time (state slots of the engine)")
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--dump-layers", default=None, metavar="DIR",
                     help="also write the residual stream at the wanted places after the embedding and after every layer "
@@ -87,7 +88,7 @@ def main(argv=None) -> int:
         os.makedirs(args.dump_layers, exist_ok=True)
     print(f"[trace_run] loading {args.model} as {args.dtype}", file=sys.stderr, flush=True)
     lm = load_model(args.model, dtype=args.dtype, device=args.device, page_size=args.page_size,
-                    max_tokens=args.max_tokens, max_requests=64)
+                    max_tokens=args.max_tokens, max_requests=args.max_requests)
     print("[trace_run] ready", file=sys.stderr, flush=True)
 
     def say(msg):

@@ -1,7 +1,9 @@
 """Builds the HIP libraries for gfx950 with hipcc, in-tree, and finds them again.
 
 One "core" library per element type (matrix products, norms, rotation and cache write,
-embedding, sampling) and one attention library per element type and head-size tile.  A
+embedding, sampling), one attention library per element type and head-size tile, and one
+library per element type for the mixers with state of fixed size ("recurrent") and for the
+attention whose heads exchange scores ("talking"), which only the models that have them load.  A
 library is rebuilt when the hash of its sources and flags differs from the stamp beside it,
 so a fresh checkout compiles at its first call exactly the libraries the model at hand
 needs, and prints a line now and then while it does.
@@ -64,9 +66,14 @@ def _hipcc() -> str:
     raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin): the HIP kernels cannot be built")
 
 
+EXTRA_KINDS = {"recurrent": "recurrent.hip", "talking": "talking.hip"}  # libraries that only some models load
+
+
 def _sources_of(kind: str):
     if kind == "core":
         return list(CORE_SOURCES)
+    if kind in EXTRA_KINDS:
+        return ["errors.hip", EXTRA_KINDS[kind]]
     return ["errors.hip", "attention.hip"]
 
 
@@ -222,6 +229,8 @@ def build_all(force: bool = True, workers: int = 4) -> list:
     jobs = []
     for elem in ELEM_DEFINE:
         jobs.append(("core", elem, None))
+        for kind in EXTRA_KINDS:
+            jobs.append((kind, elem, None))
         for nd in ATTENTION_TILES:
             jobs.append(("attention", elem, nd))
     with ThreadPoolExecutor(max_workers=workers) as pool:

@@ -62,6 +62,7 @@ class HipOps:
         self._libs: list = []
         self._core = self._load(build.ensure_library("core", self.elem))
         self._attn = {}
+        self._extra: dict = {}  # libraries that only some models need, loaded (and built) when first asked for
         self._cus = torch.cuda.get_device_properties(self._index).multi_processor_count
         # what the library plans for a product depends on its sizes alone: asked once per size
         self._plans: dict = {}
@@ -536,6 +537,193 @@ class HipOps:
         self._check(lib, fn(_ptr(q), _ptr(kpool), _ptr(vpool), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(block_table),
                             _c_int(block_table.shape[1]), _ptr(seq_pos0), _c_int(S), _c_int(H), _c_int(KV), _c_int(hd),
                             _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ a branch's output, normalised, into the stream
+    def norm_add(self, x: torch.Tensor, partials: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+        """``x += rmsnorm(sum(partials)) * weight``: ``partials`` float32 ``[P, T, d]`` are the sums of a branch's last
+        product (see :meth:`linear_split`)."""
+        T, d = x.shape
+        self._want(x, torch.float32, "norm_add stream")
+        self._want(partials, torch.float32, "norm_add sums", partials.shape[0], T, d)
+        self._want(weight, torch.float32, "norm_add weight", d)
+        self._check(self._core, self._core.ms_norm_add(_ptr(x), _ptr(partials), _c_int(partials.shape[0]), _ptr(weight), _c_int(T),
+                                                       _c_int(d), _c_float(eps), self._stream()))
+
+    def softcap(self, logits: torch.Tensor, scale: float, cap: float) -> None:
+        """In place ``v = logits * scale``, then ``cap * tanh(v / cap)`` (``cap`` 0: ``v`` as it is)."""
+        self._want(logits, torch.float32, "softcap logits")
+        self._check(self._core, self._core.ms_softcap(_ptr(logits), ctypes.c_long(logits.numel()), _c_float(scale), _c_float(cap),
+                                                      self._stream()))
+
+    # ------------------------------------------------------------------ mixers with state of fixed size
+    def _extra_lib(self, kind: str):
+        lib = self._extra.get(kind)
+        if lib is None:
+            lib = self._extra[kind] = self._load(build.ensure_library(kind, self.elem))
+        return lib
+
+    def _seq_operands(self, what, seq_q_start, seq_q_len, seq_slot):
+        S = seq_q_start.numel()
+        for t, n in ((seq_q_start, "seq_q_start"), (seq_q_len, "seq_q_len"), (seq_slot, "seq_slot")):
+            self._want(t, torch.int32, f"{what} {n}", S)
+        return S
+
+    def recurrent_limits(self) -> dict:
+        """The largest sizes the kernels of the mixers with state take."""
+        lib = self._extra_lib("recurrent")
+        return {"taps": lib.ms_conv_max_taps(), "states": lib.ms_scan_max_states(), "lightning_dim": lib.ms_lightning_max_dim()}
+
+    def causal_conv(self, xz: torch.Tensor, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+                    seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor) -> torch.Tensor:
+        """``silu(bias + causal convolution)`` per channel of the first ``channels`` columns of ``xz [T, ld]``, a request's
+        earlier inputs coming from ``state [slots, taps - 1, channels]`` (float32), which is brought up to date."""
+        lib = self._extra_lib("recurrent")
+        T, ld = xz.shape
+        taps = weight.shape[1]
+        self._want(xz, self.dtype, "convolution input")
+        self._want(weight, torch.float32, "convolution weight", channels, taps)
+        if bias is not None:
+            self._want(bias, torch.float32, "convolution bias", channels)
+        self._want(state, torch.float32, "convolution state", state.shape[0], max(taps - 1, 1), channels)
+        S = self._seq_operands("convolution", seq_q_start, seq_q_len, seq_slot)
+        out = torch.empty((T, channels), dtype=self.dtype, device=xz.device)
+        self._check(lib, lib.ms_causal_conv(_ptr(xz), _c_int(ld), _ptr(weight), _ptr(bias), _ptr(state), _ptr(seq_q_start),
+                                            _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(out), _c_int(T), _c_int(channels),
+                                            _c_int(taps), self._stream()))
+        return out
+
+    def selective_scan(self, x: torch.Tensor, xz: torch.Tensor, dbc: torch.Tensor, dt_rank: int, n_states: int, w_dt: torch.Tensor,
+                       b_dt: Optional[torch.Tensor], a_log: torch.Tensor, d_skip: Optional[torch.Tensor], state: torch.Tensor,
+                       seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor) -> torch.Tensor:
+        """The scan of a Mamba layer over the step's rows.  ``x [T, C]``: the convolved input; ``xz [T, 2 C]``: its second
+        half is the gate; ``dbc`` float32 ``[T, dt_rank + 2 n_states]``: step size input, B and C.  Step sizes are
+        ``softplus(w_dt @ low + b_dt)``; ``state`` float32 ``[slots, C, n_states]`` is carried on.  Returns
+        ``y * silu(gate)`` ``[T, C]``."""
+        lib = self._extra_lib("recurrent")
+        T, C = x.shape
+        self._want(x, self.dtype, "scan input")
+        self._want(xz, self.dtype, "scan gate", T, 2 * C)
+        self._want(dbc, torch.float32, "scan step input", T, dt_rank + 2 * n_states)
+        self._want(w_dt, torch.float32, "scan step weight", C, dt_rank)
+        if b_dt is not None:
+            self._want(b_dt, torch.float32, "scan step bias", C)
+        self._want(a_log, torch.float32, "scan A_log", C, n_states)
+        if d_skip is not None:
+            self._want(d_skip, torch.float32, "scan D", C)
+        self._want(state, torch.float32, "scan state", state.shape[0], C, n_states)
+        S = self._seq_operands("scan", seq_q_start, seq_q_len, seq_slot)
+        dt = torch.empty((T, C), dtype=torch.float32, device=x.device)
+        ldb = dbc.shape[1]
+        self._check(lib, lib.ms_dt_softplus(_ptr(dbc), _c_int(ldb), _ptr(w_dt), _ptr(b_dt), _ptr(dt), _c_int(T), _c_int(C),
+                                            _c_int(dt_rank), self._stream()))
+        y = torch.empty((T, C), dtype=self.dtype, device=x.device)
+        z = _c_void(xz.data_ptr() + C * xz.element_size())
+        self._check(lib, lib.ms_selective_scan(_ptr(x), z, _c_int(2 * C), _ptr(dt), _ptr(dbc), _c_int(ldb), _c_int(dt_rank),
+                                               _c_int(dt_rank + n_states), _ptr(a_log), _ptr(d_skip), _ptr(state), _ptr(seq_q_start),
+                                               _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(y), _c_int(T), _c_int(C),
+                                               _c_int(n_states), self._stream()))
+        return y
+
+    def lightning_attention(self, qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.Tensor, state: torch.Tensor,
+                            seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor) -> torch.Tensor:
+        """Linear attention with a decay per head over the step's rows.  ``qkvg [T, ld]`` holds q ``[heads, dim]``, k
+        ``[heads, dim]``, v ``[heads, vdim]`` (and whatever follows) before their SiLU; ``state`` float32
+        ``[slots, heads, dim, vdim]`` is carried on.  Returns float32 ``[T, heads * vdim]``."""
+        lib = self._extra_lib("recurrent")
+        T, ld = qkvg.shape
+        self._want(qkvg, self.dtype, "lightning q/k/v")
+        self._want(decay, torch.float32, "lightning decay", heads)
+        self._want(state, torch.float32, "lightning state", state.shape[0], heads, dim, vdim)
+        S = self._seq_operands("lightning", seq_q_start, seq_q_len, seq_slot)
+        o = torch.empty((T, heads * vdim), dtype=torch.float32, device=qkvg.device)
+        self._check(lib, lib.ms_lightning(_ptr(qkvg), _c_int(ld), _c_int(0), _c_int(heads * dim), _c_int(2 * heads * dim), _ptr(decay),
+                                          _ptr(state), _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(o),
+                                          _c_int(T), _c_int(heads), _c_int(dim), _c_int(vdim), self._stream()))
+        return o
+
+    def gated_rmsnorm(self, o: torch.Tensor, gate_of: torch.Tensor, gate_col: int, weight: torch.Tensor, eps: float) -> torch.Tensor:
+        """``rmsnorm(o) * weight * sigmoid(gate)`` in the element type; the gate is columns ``gate_col`` onwards of
+        ``gate_of [T, ld]``."""
+        lib = self._extra_lib("recurrent")
+        T, n = o.shape
+        self._want(o, torch.float32, "gated norm input")
+        self._want(gate_of, self.dtype, "gated norm gate")
+        if gate_of.shape[0] != T or gate_col < 0 or gate_col + n > gate_of.shape[1]:
+            raise KernelError(f"gated norm: gate columns {gate_col}..{gate_col + n} of {tuple(gate_of.shape)} for {T} rows")
+        self._want(weight, torch.float32, "gated norm weight", n)
+        out = torch.empty((T, n), dtype=self.dtype, device=o.device)
+        gate = _c_void(gate_of.data_ptr() + gate_col * gate_of.element_size())
+        self._check(lib, lib.ms_gated_rmsnorm(_ptr(o), gate, _c_int(gate_of.shape[1]), _ptr(weight), _ptr(out), _c_int(T), _c_int(n),
+                                              _c_float(eps), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ attention whose heads exchange scores
+    def talking_limits(self) -> dict:
+        return {"row": self._extra_lib("talking").ms_talking_max_row()}
+
+    def talking_prepare(self, qkv: torch.Tensor, q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float,
+                        positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rot: int, cs_factor: float,
+                        v_other: Optional[torch.Tensor], v_lambda: Optional[torch.Tensor], keep_values: bool, slot_map: torch.Tensor,
+                        kpool: torch.Tensor, vpool: torch.Tensor, H: int, KV: int, d: int, dv: int, page_size: int):
+        """Finishes the rows of a q/k/v product given as float32 partial sums ``[P, T, stride]`` (q ``[H, d]``, k
+        ``[KV, d]``, v ``[KV, dv]``): RMS norm over the whole of q and of k (weights ``q_norm``, ``k_norm``; None: no
+        norm), rotation of the first ``rot`` numbers of every head by ``positions * inv_freq`` with cosines and sines
+        times ``cs_factor``, values blended as ``(1 - v_lambda) v + v_lambda v_other``, keys and values written to their
+        pages.  Returns ``(q [T, H * d]`` in the element type, the rows' own values float32 ``[T, KV * dv]`` before the
+        blend if ``keep_values`` else None)``."""
+        lib = self._extra_lib("talking")
+        if qkv.dim() == 2:
+            qkv = qkv.unsqueeze(0)
+        P, T, stride = qkv.shape
+        self._want(qkv, torch.float32, "attention rows")
+        if q_norm is not None:
+            self._want(q_norm, torch.float32, "query norm weight", H * d)
+        if k_norm is not None:
+            self._want(k_norm, torch.float32, "key norm weight", KV * d)
+        self._want(positions, torch.int32, "attention positions", T)
+        if inv_freq is not None:
+            self._want(inv_freq, torch.float32, "attention inv_freq", rot // 2)
+        if v_other is not None:
+            self._want(v_other, torch.float32, "values to blend with", T, KV * dv)
+            self._want(v_lambda, torch.float32, "blend weight")
+        self._want(slot_map, torch.int32, "attention slot_map", T)
+        pages = kpool.shape[0]
+        self._want(kpool, self.dtype, "key pool", pages, KV, page_size, d)
+        self._want(vpool, self.dtype, "value pool", pages, KV, dv, page_size)
+        q = torch.empty((T, H * d), dtype=self.dtype, device=qkv.device)
+        v_raw = torch.empty((T, KV * dv), dtype=torch.float32, device=qkv.device) if keep_values else None
+        self._check(lib, lib.ms_talking_prepare(
+            _ptr(qkv), _c_int(P), _c_int(stride), _ptr(q_norm), _ptr(k_norm), _c_float(eps), _ptr(positions), _ptr(inv_freq), _c_int(rot),
+            _c_float(cs_factor), _ptr(v_other), _ptr(v_lambda), _ptr(v_raw), _ptr(slot_map), _ptr(q), _ptr(kpool), _ptr(vpool), _c_int(T),
+            _c_int(H), _c_int(KV), _c_int(d), _c_int(dv), _c_int(page_size), self._stream()))
+        return q, v_raw
+
+    def talking_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, talk: Optional[torch.Tensor],
+                          block_table: torch.Tensor, seq_q_start: torch.Tensor, seq_pos0: torch.Tensor, H: int, KV: int, d: int, dv: int,
+                          page_size: int, window: Optional[int], keep_first: int, scale: float) -> torch.Tensor:
+        """Attention of every row over the keys it sees: the last ``window`` positions up to its own (None: all) and
+        the request's first ``keep_first``.  ``talk`` float32 ``[H, H]`` mixes the heads' scaled scores before the
+        softmax (None: no exchange).  Returns ``[T, H * dv]`` in the element type."""
+        lib = self._extra_lib("talking")
+        T = q.shape[0]
+        self._want(q, self.dtype, "attention q", T, H * d)
+        pages = kpool.shape[0]
+        self._want(kpool, self.dtype, "key pool", pages, KV, page_size, d)
+        self._want(vpool, self.dtype, "value pool", pages, KV, dv, page_size)
+        if talk is not None:
+            self._want(talk, torch.float32, "head exchange", H, H)
+        S = seq_q_start.numel()
+        self._want(block_table, torch.int32, "block table")
+        if block_table.dim() != 2 or block_table.shape[0] != S:
+            raise KernelError(f"attention: block table {tuple(block_table.shape)} for {S} requests")
+        self._want(seq_q_start, torch.int32, "seq_q_start", S)
+        self._want(seq_pos0, torch.int32, "seq_pos0", S)
+        out = torch.empty((T, H * dv), dtype=self.dtype, device=q.device)
+        self._check(lib, lib.ms_talking_attention(
+            _ptr(q), _ptr(kpool), _ptr(vpool), _ptr(talk), _ptr(block_table), _c_int(block_table.shape[1]), _ptr(seq_q_start),
+            _ptr(seq_pos0), _c_int(S), _ptr(out), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv), _c_int(page_size),
+            _c_int(window or 0), _c_int(keep_first), _c_float(scale), self._stream()))
         return out
 
     # ------------------------------------------------------------------ sampling

@@ -44,6 +44,7 @@ class PagedKVRequest:
     head_dim: int
     window: Optional[int] = None
     v_head_dim: Optional[int] = None
+    keep_first: int = 0  # with a window: the request's first tokens stay visible (and their pages are never given back)
 
 
 @dataclass(frozen=True)

@@ -1,4 +1,5 @@
-"""Arrangements of parts in a block.  Pre-norm (``crates/mach-model/src/batched.rs:3180-3200,
+"""Arrangements of parts in a block.  Sandwich: a norm before and one after each branch,
+``x += post(mixer(pre(x))); x += post(feed_forward(pre(x)))``.  Pre-norm (``crates/mach-model/src/batched.rs:3180-3200,
 4031, 4050, 4453``): ``x += mixer(norm(x)); x += feed_forward(norm(x))``."""
 from __future__ import annotations
 
@@ -33,3 +34,56 @@ class PreNormBlock(Block):
             if pending is not None:
                 return pending
         return norm.forward(stream)
+
+
+class _Branch:
+    """What a branch of a sandwich block writes to in the stream's place: it keeps the branch's output, as the
+    operands of its last product or as a finished tensor, for the norm that follows."""
+
+    def __init__(self, ops):
+        self.ops = ops
+        self.product = None
+        self.tensor = None
+
+    def add_linear(self, a, w) -> None:
+        self.product = (a, w)
+
+    def add(self, y) -> None:
+        self.tensor = y
+
+
+@register_block("sandwich")
+class SandwichBlock(Block):
+    """Reads ``mixer``, ``feed_forward`` (may be None), ``mixer_norm``, ``mixer_post_norm``, ``feed_forward_norm`` and
+    ``feed_forward_post_norm`` of its layer's spec.  A post norm is a norm with ``add_normed``."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.mixer = MIXERS.build(spec.mixer, rt)
+        self.mixer_norm = NORMS.build(spec.mixer_norm, rt)
+        self.mixer_post_norm = NORMS.build(spec.mixer_post_norm, rt)
+        self.feed_forward = self.feed_forward_norm = self.feed_forward_post_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, rt)
+            self.feed_forward_norm = NORMS.build(spec.feed_forward_norm, rt)
+            self.feed_forward_post_norm = NORMS.build(spec.feed_forward_post_norm, rt)
+
+    def parts(self):
+        out = [self.mixer_norm, self.mixer, self.mixer_post_norm]
+        if self.feed_forward is not None:
+            out += [self.feed_forward_norm, self.feed_forward, self.feed_forward_post_norm]
+        return out
+
+    def forward(self, stream, ctx):
+        self._branch(self.mixer_norm, self.mixer, self.mixer_post_norm, stream, ctx)
+        if self.feed_forward is not None:
+            self._branch(self.feed_forward_norm, self.feed_forward, self.feed_forward_post_norm, stream, ctx)
+
+    def _branch(self, pre, part, post, stream, ctx):
+        out = _Branch(self.rt.ops)
+        part.forward(PreNormBlock._input(pre, part, stream), out, ctx)
+        stream.flush()  # a norm left pending has added what was pending by now; nothing else may be
+        if out.product is not None:
+            post.add_normed(stream, *out.product)
+        else:
+            post.add_normed_tensor(stream, out.tensor)

@@ -30,7 +30,7 @@ class Embedding(Part):
 
 @register_head("linear")
 class Head(Part):
-    """Output projection, times the spec's ``scale``; tied to the embedding table when the spec says so, or
+    """Output projection, times the spec's ``scale``, then capped by a tanh if the spec has a ``softcap``; tied to the embedding table when the spec says so, or
     when it leaves it open and the checkpoint has no head tensor
     (``crates/mach-model/src/loader.rs:1025-1033``).  A head is built with the model's embedding part as
     its third argument and has ``forward(h) -> float32 logits`` and ``vocab`` in its spec."""
@@ -55,8 +55,10 @@ class Head(Part):
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         w = self.weight if self.weight is not None else self.embedding.weight
         logits = self.rt.ops.linear(h, w, None, out_f32=True)
-        scale = getattr(self.spec, "scale", 1.0)
-        if scale != 1.0:
+        scale, cap = getattr(self.spec, "scale", 1.0), getattr(self.spec, "softcap", 0.0)
+        if cap:
+            self.rt.ops.softcap(logits, scale, cap)  # scale, then cap * tanh(. / cap), in one pass
+        elif scale != 1.0:
             logits *= scale
         return logits
 

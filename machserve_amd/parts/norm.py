@@ -31,6 +31,30 @@ class RMSNorm(Norm):
     def pending(self, stream):
         return PendingRMSNorm(self, stream)
 
+    def add_normed(self, stream, a, w) -> None:
+        """``x += rmsnorm(a @ w.T) * weight``: the norm after a branch whose last step is a product.  The product
+        leaves its sums in 32-bit, and one kernel adds them up, normalises the row and adds it to the stream."""
+        stream.flush()
+        stream.ops.norm_add(stream.x, stream.ops.linear_split(a, w), self.weight, self.spec.eps)
+
+    def add_normed_tensor(self, stream, y) -> None:
+        """``x += rmsnorm(y) * weight`` for a branch that computes its output by other means."""
+        stream.flush()
+        stream.ops.norm_add(stream.x, y.float().contiguous().unsqueeze(0), self.weight, self.spec.eps)
+
+
+@register_norm("rmsnorm_scalar")
+class ScalarRMSNorm(RMSNorm):
+    """RMS norm whose weight is one number for all coordinates: ``y = x / sqrt(mean(x^2) + eps) * g``.  The number is
+    spread over the width when it is loaded, so every kernel and every folded form of the norm with a weight per
+    coordinate serves it."""
+
+    def tensor_decls(self):
+        return [TensorDecl("weight", (), "vector")]
+
+    def load(self, tensors):
+        self.weight = tensors["weight"].reshape(1).expand(self.spec.width).contiguous()
+
 
 class PendingRMSNorm(PendingNorm):
     """The RMS norm left to its reader's first product, folded into it where the kernels take the shape."""

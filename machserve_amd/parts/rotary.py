@@ -24,29 +24,35 @@ _TABLES = weakref.WeakValueDictionary()
 class Rotary(PositionEncoding):
     def __init__(self, spec, rt):
         super().__init__(spec, rt)
-        hd = spec.head_dim
-        j = torch.arange(hd // 2, dtype=torch.float32)
-        theta = torch.tensor(float(spec.theta), dtype=torch.float32)
+        # a rotation of the first `rotary_dim` numbers of a head takes its frequencies and YaRN's bounds from that size
+        hd = self.rotary_dim = getattr(spec, "rotary_dim", None) or spec.head_dim
+        if hd % 2 or hd > spec.head_dim:
+            raise ValueError(f"rotary: {hd} of {spec.head_dim} numbers of a head cannot be rotated in pairs")
+        # the table is made in this precision and rounded to 32-bit once, at the end
+        real = {"float32": torch.float32, "float64": torch.float64}[getattr(spec, "table_precision", "float32")]
+        j = torch.arange(hd // 2, dtype=real)
+        theta = torch.tensor(float(spec.theta), dtype=real)
         inv = 1.0 / torch.pow(theta, 2.0 * j / hd)
         self.factor = 1.0
         yarn = getattr(spec, "yarn", None)
         if yarn is not None:
             # Between pair indices `low` and `high` a frequency goes over from its own value to 1 / factor of it; the
             # bounds are where beta_fast and beta_slow rotations fit the original context, clamped to the head size
-            # (not to the number of pairs), every step in 32-bit as the reference takes it.
-            f32 = lambda v: torch.tensor(float(v), dtype=torch.float32)
+            # (not to the number of pairs), every step in the table's precision (32-bit as the reference takes it).
+            f32 = lambda v: torch.tensor(float(v), dtype=real)
             two_ln_theta = 2.0 * torch.log(theta)
 
             def pair_of(rotations):
                 return hd * torch.log(f32(yarn.original_max_positions) / (f32(rotations) * 2.0 * f32(math.pi))) / two_ln_theta
             low = max(float(torch.floor(pair_of(yarn.beta_fast))), 0.0)
             high = min(float(torch.ceil(pair_of(yarn.beta_slow))), hd - 1.0)
-            if high == low:
-                high += 0.001
+            if high <= low:  # no ramp but a step: everything from `low` on is scaled
+                high = low + 0.001
             ramp = ((j - low) / (f32(high) - f32(low))).clamp(0.0, 1.0)
             inv = (1.0 / (f32(yarn.factor) * torch.pow(theta, 2.0 * j / hd))) * ramp + inv * (1.0 - ramp)
             ln = math.log(yarn.factor)
             self.factor = (0.1 * yarn.mscale * ln + 1.0) / (0.1 * yarn.mscale_all_dim * ln + 1.0)
+        inv = inv.to(torch.float32)
         key = (str(rt.device), inv.numpy().tobytes())
         table = _TABLES.get(key)
         if table is None:

@@ -22,12 +22,27 @@ STD = 0.02
 
 
 def _draw(shape, law: str, gen: torch.Generator, device) -> torch.Tensor:
-    t = torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * STD
-    if law == "norm":
-        t = t + 1.0
-    elif law not in ("matrix", "bias"):
-        raise ValueError(f"unknown law {law!r}")
-    return t
+    """One tensor of a law.  Beside the three above: 'filter' ~ N(0, 0.3) (a short convolution, a narrow projection
+    inside a recurrence); 'mixing' = identity + N(0, 0.1) (a square matrix that mixes heads); 'blend' ~ U(0.3, 0.7) (a
+    weight between two tensors); 'a_log' = ln(1 .. n) along the last axis (the decays of a scan); 'step_bias': the
+    inverse softplus of step sizes drawn log-uniformly from 0.001 to 0.1."""
+    if law in ("matrix", "bias", "norm"):
+        t = torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * STD
+        return t + 1.0 if law == "norm" else t
+    if law == "filter":
+        return torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * 0.3
+    if law == "mixing":
+        return torch.eye(shape[0], shape[1], device=device) + torch.randn(shape, generator=gen, dtype=torch.float32, device=device) * 0.1
+    if law == "blend":
+        return 0.3 + 0.4 * torch.rand(shape, generator=gen, dtype=torch.float32, device=device)
+    if law == "a_log":
+        return torch.log(torch.arange(1, shape[-1] + 1, dtype=torch.float32, device=device)).expand(shape).clone()
+    if law == "step_bias":
+        import math
+        u = torch.rand(shape, generator=gen, dtype=torch.float32, device=device)
+        dt = torch.exp(u * (math.log(0.1) - math.log(0.001)) + math.log(0.001))
+        return dt + torch.log(-torch.expm1(-dt))
+    raise ValueError(f"unknown law {law!r}")
 
 
 def random_tensors(config, seed: int, dtype: torch.dtype = torch.float32,

@@ -184,3 +184,126 @@ class EmulatedOps:
     def logit_edit(self, logits, row_of, token, delta):
         for r, t, d in zip(row_of.tolist(), token.tolist(), delta.tolist()):
             logits[r, t] += d
+
+    # ------------------------------------------------------------------ a branch's output, normalised, into the stream
+    def norm_add(self, x, partials, weight, eps):
+        y = partials.sum(0)
+        x += y * (1.0 / torch.sqrt((y * y).sum(-1, keepdim=True) / y.shape[-1] + eps)) * weight
+
+    def softcap(self, logits, scale, cap):
+        v = logits * scale
+        logits.copy_(cap * torch.tanh(v / cap) if cap > 0 else v)
+
+    # ------------------------------------------------------------------ mixers with state of fixed size
+    def recurrent_limits(self):
+        return {"taps": 16, "states": 128, "lightning_dim": 256}
+
+    def causal_conv(self, xz, channels, weight, bias, state, seq_q_start, seq_q_len, seq_slot):
+        taps = weight.shape[1]
+        out = torch.empty(xz.shape[0], channels)
+        for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
+            x = xz[q0:q0 + n, :channels].float()
+            hist = torch.cat([state[slot][:taps - 1], x], 0)       # the taps - 1 inputs before, then the step's
+            acc = torch.zeros(n, channels) if bias is None else bias.expand(n, channels).clone()
+            for k in range(taps):
+                acc += hist[k:k + n] * weight[:, k]
+            out[q0:q0 + n] = _act(acc, "silu")
+            if taps > 1:
+                state[slot][:taps - 1] = hist[n:]
+        return self._r(out)
+
+    def selective_scan(self, x, xz, dbc, dt_rank, n_states, w_dt, b_dt, a_log, d_skip, state, seq_q_start, seq_q_len, seq_slot):
+        T, C = x.shape
+        low, B, Cm = dbc[:, :dt_rank], dbc[:, dt_rank:dt_rank + n_states], dbc[:, dt_rank + n_states:]
+        dt = torch.nn.functional.softplus(low @ w_dt.t() + (0 if b_dt is None else b_dt))
+        A = -torch.exp(a_log)
+        xf, z = x.float(), xz[:, C:].float()
+        y = torch.empty(T, C)
+        for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
+            S = state[slot].clone()
+            for t in range(q0, q0 + n):
+                S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * xf[t])[:, None] * B[t][None, :]
+                y[t] = S @ Cm[t] + (0 if d_skip is None else d_skip * xf[t])
+            state[slot] = S
+        return self._r(y * _act(z, "silu"))
+
+    def lightning_attention(self, qkvg, heads, dim, vdim, decay, state, seq_q_start, seq_q_len, seq_slot):
+        T = qkvg.shape[0]
+        f = qkvg.float()
+        q = _act(f[:, :heads * dim], "silu").view(T, heads, dim)
+        k = _act(f[:, heads * dim:2 * heads * dim], "silu").view(T, heads, dim)
+        v = _act(f[:, 2 * heads * dim:2 * heads * dim + heads * vdim], "silu").view(T, heads, vdim)
+        o = torch.empty(T, heads, vdim)
+        for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
+            S = state[slot].clone()
+            for t in range(q0, q0 + n):
+                S = decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+                o[t] = torch.einsum("hde,hd->he", S, q[t])
+            state[slot] = S
+        return o.reshape(T, heads * vdim)
+
+    def gated_rmsnorm(self, o, gate_of, gate_col, weight, eps):
+        n = o.shape[1]
+        g = gate_of[:, gate_col:gate_col + n].float()
+        return self._r(o * (1.0 / torch.sqrt((o * o).sum(-1, keepdim=True) / n + eps)) * weight * torch.sigmoid(g))
+
+    # ------------------------------------------------------------------ attention whose heads exchange scores
+    def talking_limits(self):
+        return {"row": 15000}
+
+    def talking_prepare(self, qkv, q_norm, k_norm, eps, positions, inv_freq, rot, cs_factor, v_other, v_lambda, keep_values,
+                        slot_map, kpool, vpool, H, KV, d, dv, page_size):
+        qkv = qkv if qkv.dim() == 2 else qkv.sum(0)
+        T = qkv.shape[0]
+        nq, nk, nv = H * d, KV * d, KV * dv
+        q, k, v = qkv[:, :nq], qkv[:, nq:nq + nk], qkv[:, nq + nk:nq + nk + nv]
+        if q_norm is not None:
+            q = q * (1.0 / torch.sqrt((q * q).sum(-1, keepdim=True) / nq + eps)) * q_norm
+        if k_norm is not None:
+            k = k * (1.0 / torch.sqrt((k * k).sum(-1, keepdim=True) / nk + eps)) * k_norm
+        own = v.clone() if keep_values else None
+        if v_other is not None:
+            v = (1.0 - v_lambda[0]) * v + v_lambda[0] * v_other
+        half = rot // 2 if inv_freq is not None else 0
+
+        def rotated(x, heads):
+            x = x.reshape(T, heads, d)
+            if not half:
+                return x
+            ang = positions.float()[:, None] * inv_freq[None, :]
+            c, s = (torch.cos(ang) * cs_factor)[:, None, :], (torch.sin(ang) * cs_factor)[:, None, :]
+            a, b = x[..., :half], x[..., half:2 * half]
+            return torch.cat([a * c - b * s, b * c + a * s, x[..., 2 * half:]], -1)
+
+        q = self._r(rotated(q, H)).reshape(T, nq)
+        k = self._r(rotated(k, KV))
+        v = self._r(v).reshape(T, KV, dv)
+        page, off = (slot_map // page_size).long(), (slot_map % page_size).long()
+        for t in range(T):
+            kpool[page[t], :, off[t], :] = k[t]
+            vpool[page[t], :, :, off[t]] = v[t]
+        return q, own
+
+    def talking_attention(self, q, kpool, vpool, talk, block_table, seq_q_start, seq_pos0, H, KV, d, dv, page_size, window,
+                          keep_first, scale):
+        T, S = q.shape[0], seq_q_start.numel()
+        rep = H // KV
+        out = torch.zeros(T, H, dv)
+        starts = seq_q_start.tolist() + [T]
+        for s in range(S):
+            for t in range(starts[s], starts[s + 1]):
+                pos = int(seq_pos0[s]) + t - starts[s]
+                lo = max(0, pos - window + 1) if window else 0
+                keys = torch.tensor(list(range(min(keep_first, lo))) + list(range(lo, pos + 1)))
+                pages = block_table[s].long()[keys // page_size]
+                assert (pages >= 0).all(), "attention reads a page that was given back"
+                offs = keys % page_size
+                kk = kpool[pages, :, offs, :].float()           # [keys, KV, d]
+                vv = vpool[pages, :, :, offs].float()           # [keys, KV, dv]
+                qq = q[t].float().view(H, d) * scale
+                sc = torch.einsum("hd,jhd->hj", qq, kk.repeat_interleave(rep, dim=1))
+                if talk is not None:
+                    sc = talk @ sc
+                p = torch.softmax(sc, -1)
+                out[t] = torch.einsum("hj,jhe->he", p, vv.repeat_interleave(rep, dim=1))
+        return self._r(out.reshape(T, H * dv))
