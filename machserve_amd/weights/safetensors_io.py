@@ -117,4 +117,4 @@ def write_safetensors(path: str, plan: Iterable[Tuple[str, Tuple[int, ...], torc
             if tuple(t.shape) != tuple(shape) or t.dtype != dtype:
                 raise SafetensorsError(f"{name}: produced {tuple(t.shape)} {t.dtype}, planned {tuple(shape)} {dtype}")
             t = t.contiguous().cpu()
-            f.write(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"")
+            f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b"")  # (a single number has no axis to view along)

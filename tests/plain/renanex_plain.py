@@ -173,9 +173,9 @@ def forward(weights, cfg, tokens, dtype=torch.float64, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     h = rms(x, eps) * weights["final.norm"].to(dtype)
-    logits = (h @ weights["head"].to(dtype).T) * float(cfg["logit_scale"])
-    cap = float(cfg["logit_softcap"])
-    return cap * torch.tanh(logits / cap)
+    logits = (h @ weights["head"].to(dtype).T) * float(cfg.get("logit_scale", 1.0))
+    cap = float(cfg.get("logit_softcap") or 0.0)
+    return cap * torch.tanh(logits / cap) if cap else logits
 
 
 def greedy_generate(weights, cfg, prompt, max_new, dtype=torch.float64):
