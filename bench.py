@@ -268,6 +268,92 @@ def build_probe(dtype_name, force=False):
     return build.ensure_extra_library("bench_mfma_probe", dtype_name, os.path.join(here, "bench_mfma_probe.hip"), force)
 
 
+# ---- Renanex beside Qwen2 at equal sizes ---------------------------------------------------
+# width, feed-forward, heads, key/value heads, head size, window, layers (a multiple of four: Renanex runs them as
+# scan, attention, attention, lightning), prompt tokens, decode batch, decode context
+DESIGN_SIZES = {
+    "small": dict(width=1024, ff=2816, heads=8, kv=2, hd=128, window=512, layers=4, prompt=2048, batch=8, context=1024),
+    "medium": dict(width=2048, ff=5632, heads=16, kv=4, hd=128, window=1024, layers=4, prompt=2048, batch=16, context=2048),
+    "large": dict(width=4096, ff=11008, heads=32, kv=8, hd=128, window=2048, layers=4, prompt=4096, batch=32, context=2048),
+}
+DESIGN_VOCAB = 32000
+
+
+def design_configs(z):
+    """(Renanex configuration, Qwen2 configuration) of one size, as config.json dicts."""
+    w, H, kv, hd = z["width"], z["heads"], z["kv"], z["hd"]
+    att = {"type": "attention", "mlp": {"kind": "dense", "ff": z["ff"]},
+           "mixer": {"heads": H, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "v_mix": True,
+                     "mask": {"size": z["window"], "keep_first": 4},
+                     "rot": {"base": 10000.0, "dims": hd, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    scan = {"type": "mamba1", "mlp": {"kind": "dense", "ff": z["ff"]},
+            "mixer": {"inner": 2 * w, "state": 16, "dt_rank": w // 16, "conv": 4}}
+    lin = {"type": "lightning", "mlp": {"kind": "dense", "ff": z["ff"]},
+           "mixer": {"heads": H, "dim": hd, "vdim": hd, "decay": [1.0 - 2.0 ** (-5 - 3 * i / max(H - 1, 1)) for i in range(H)]}}
+    renanex = {"architecture": "Renanex", "vocab": DESIGN_VOCAB, "width": w, "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+               "logit_softcap": 30.0, "layers": [scan, att, att, lin] * (z["layers"] // 4)}
+    qwen = {"architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2", "hidden_size": w, "num_hidden_layers": z["layers"],
+            "num_attention_heads": H, "num_key_value_heads": kv, "head_dim": hd, "intermediate_size": z["ff"], "vocab_size": DESIGN_VOCAB,
+            "max_position_embeddings": 32768, "rms_norm_eps": 1e-6, "rope_theta": 10000.0, "tie_word_embeddings": False,
+            "hidden_act": "silu", "use_sliding_window": True, "sliding_window": z["window"], "max_window_layers": 0}
+    return renanex, qwen
+
+
+def compare_designs(args) -> int:
+    """Prefill (one prompt in one step) and decode (a batch of single tokens at a context, from the captured step)
+    of both designs through the step function; random weights, synthetic tokens.  One JSON line."""
+    import torch
+    from machserve_amd.config import config_from_dict
+    from machserve_amd.engine import load_model
+    from machserve_amd.engine.step import StepEntry
+    from machserve_amd.weights import random_tensor_dict
+    dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[args.dtype]
+    gen = torch.Generator().manual_seed(2)
+    out = {}
+    for size in args.design_sizes.split(","):
+        z = DESIGN_SIZES[size]
+        out[size] = {"sizes": z}
+        for name, raw in zip(("renanex", "qwen2"), design_configs(z)):
+            cfg = config_from_dict(raw)
+            tensors = random_tensor_dict(cfg, 0, dt, device="cuda:0")
+            page = args.page_size
+            need = max(z["prompt"] + page, z["batch"] * (z["context"] + args.warmup + args.steps + 2 * page))
+            lm = load_model(config=cfg, tensors=tensors, dtype=dt, page_size=page, max_tokens=need, max_requests=z["batch"])
+            toks = lambda n: torch.randint(0, DESIGN_VOCAB, (n,), generator=gen).tolist()
+            times = []
+            for _ in range(lm.step.FILLED_CAPTURE_AFTER + 4):   # launched, captured, then replayed as in serving
+                slot = lm.cache.admit()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                lm.step([StepEntry(slot, toks(z["prompt"]), [z["prompt"] - 1])], borrow_logits=True)
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                lm.cache.release(slot)
+            prefill = min(times[-3:])
+            slots = [lm.cache.admit() for _ in range(z["batch"])]
+            for sl in slots:
+                lm.step([StepEntry(sl, toks(z["context"]), [])])
+            step = lambda: lm.step([StepEntry(sl, [1], [0]) for sl in slots], borrow_logits=True)
+            for _ in range(args.warmup + 2):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                step()
+            torch.cuda.synchronize()
+            decode = (time.perf_counter() - t0) / args.steps
+            out[size][name] = {"prefill_tok_s": round(z["prompt"] / prefill, 1), "prefill_ms": round(prefill * 1e3, 3),
+                               "decode_tok_s": round(z["batch"] / decode, 1), "decode_ms": round(decode * 1e3, 4)}
+            del lm, tensors
+            torch.cuda.empty_cache()
+        r, q = out[size]["renanex"], out[size]["qwen2"]
+        out[size]["renanex_over_qwen2"] = {"prefill": round(r["prefill_tok_s"] / q["prefill_tok_s"], 3),
+                                           "decode": round(r["decode_tok_s"] / q["decode_tok_s"], 3)}
+    print(json.dumps({"metric": "renanex_beside_qwen2_tokens_per_s", "dtype": args.dtype, "data": "synthetic", "steps": args.steps,
+                      "warmup": args.warmup, "sizes": out}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -288,11 +374,17 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=None, help="tokens of the prefill (default: the context)")
     ap.add_argument("--profile-out", default=None, help="folder that receives a summary of the traced runs, one text file for the decode "
                     "step and one for the prefill (kinds of kernels, and the kernels by name)")
+    ap.add_argument("--designs", action="store_true",
+                    help="instead of the default run: prefill and decode throughput of Renanex layers (Mamba scan, attention whose heads "
+                         "exchange scores over a window, lightning attention) beside Qwen2 layers of equal sizes, at a few sizes")
+    ap.add_argument("--design-sizes", default="small,medium", help="with --designs: which of the sizes to run (small, medium, large)")
     ap.add_argument("--record-calls", default=None, help=argparse.SUPPRESS)  # file that receives one step's operations (the traced run)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.designs:
+        return compare_designs(args)
 
     import torch
     from machserve_amd.config import config_from_dict
