@@ -221,6 +221,188 @@ __global__ __launch_bounds__(256) void talking_attention_kernel(TalkArgs a) {
     }
 }
 
+// ---- a tile of 16 rows on the matrix cores -------------------------------------------------
+// A block takes rows [16 b, 16 b + 16) of the step, every head; wave w takes heads [w * HPW, (w + 1) * HPW).  Keys go by
+// in tiles of NT * 16 positions.  Per tile: each wave computes S^T = K Q^T for its heads (lane l: keys (l / 16) * 4 + i
+// of a 16-key tile, query l % 16), scales it and leaves it in LDS; after a barrier it reads, for each of its heads,
+// every head's score of its own (key, query) pairs and mixes them by the exchange matrix in 32-bit; then the running
+// softmax, in which a lane belongs to one query throughout, and O^T += V^T P^T, the weights rounded to the element
+// type as an operand of that product (not at all in the 32-bit build).  Rows of several requests in one tile are
+// taken request by request: the rows of the others are masked, which leaves their sums as they are.
+constexpr float TK_NEG_BIG = -1.0e30f;
+
+template <int HPW, int ND, int NT>
+__global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a, const int* __restrict__ seq_q_len, int T) {
+    extern __shared__ float lds[];
+    const int H = a.H, d = a.d, dv = a.dv, KV = a.KV, rep = H / KV, ps = a.ps;
+    float* raw = lds;                              // [H][16 queries][NT * 16 keys]
+    float* talk_s = raw + (size_t)H * 16 * NT * 16;  // [H][H]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r16 = lane & 15, grp = lane >> 4;
+    const int r0 = blockIdx.x * 16, r_end = min(r0 + 16, T);
+    const int my_row = min(r0 + r16, T - 1);
+    const int h0 = wave * HPW;
+    const int nks = (d + 31) / 32;
+    if (a.talk)
+        for (int i = tid; i < H * H; i += blockDim.x) talk_s[i] = a.talk[i];
+    float m_run[HPW], l_run[HPW];
+    f32x4 acc[HPW][ND];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+        m_run[hh] = TK_NEG_BIG;
+        l_run[hh] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) acc[hh][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+    const elem_t* qrow = a.q + (size_t)my_row * H * d;
+    int s = seq_of_row(r0, a.seq_q_start, a.S);
+    for (; s < a.S && a.seq_q_start[s] < r_end; ++s) {
+        const int q0 = a.seq_q_start[s], qn = seq_q_len[s], p0 = a.seq_pos0[s];
+        const int ra = max(r0, q0), rb = min(r_end, q0 + qn);  // this request's rows in the tile
+        if (ra >= rb) continue;
+        const int p_lo = p0 + (ra - q0), p_hi = p0 + (rb - 1 - q0);
+        const bool mine = r0 + r16 >= ra && r0 + r16 < rb;
+        const int pos = p0 + (r0 + r16 - q0);
+        const int lo = a.window > 0 ? max(0, p_lo - a.window + 1) : 0;
+        const int n_first = min(a.keep_first, lo);
+        const int* table = a.block_table + (size_t)s * a.table_stride;
+        constexpr int BK = NT * 16;
+        const int a_end = (n_first + BK - 1) / BK;     // tiles of the first tokens: [0, a_end)
+        const int b_begin = max(a_end, lo / BK), b_end = p_hi / BK + 1;
+        const int n_tiles = a_end + (b_end - b_begin);
+        for (int it = 0; it < n_tiles; ++it) {
+            const int kt0 = (it < a_end ? it : b_begin + (it - a_end)) * BK;
+            int page[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const int lp = (kt0 + nt * 16) / ps;
+                page[nt] = lp < a.table_stride ? table[lp] : -1;
+            }
+            // ---- raw scores of this wave's heads
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) {
+                const int h = h0 + hh;
+                if (h >= H) break;
+                const int kvh = h / rep;
+                f32x4 sc[NT];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    sc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                    const int pg = max(page[nt], 0), off = (kt0 + nt * 16) % ps;
+                    const elem_t* krow = a.kpool + (((size_t)pg * KV + kvh) * ps + off + r16) * d;
+                    for (int ks = 0; ks < nks; ++ks) {
+                        const int d0 = ks * 32 + grp * 8;
+                        const Frag kf = d0 < d ? frag_load(krow + d0) : frag_zero();
+                        const Frag qf = d0 < d ? frag_load(qrow + (size_t)h * d + d0) : frag_zero();
+                        mma_16x16x32(sc[nt], kf, qf);
+                    }
+                    if (a.talk) {
+                        float* dst = raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4;
+                        *reinterpret_cast<f32x4*>(dst) = sc[nt] * a.scale;
+                    }
+                }
+                if (!a.talk) {  // no exchange: the head's own scores stay in registers (see below)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        float* dst = raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4;
+                        *reinterpret_cast<f32x4*>(dst) = sc[nt] * a.scale;
+                    }
+                }
+            }
+            __syncthreads();
+            // ---- exchange, softmax, values
+#pragma unroll
+            for (int hh = 0; hh < HPW; ++hh) {
+                const int h = h0 + hh;
+                if (h >= H) break;
+                const int kvh = h / rep;
+                f32x4 mixed[NT];
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) mixed[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                if (a.talk) {
+                    for (int g = 0; g < H; ++g) {
+                        const float w = talk_s[h * H + g];
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+                            mixed[nt] += w * *reinterpret_cast<const f32x4*>(raw + (((size_t)g * 16 + r16) * NT + nt) * 16 + grp * 4);
+                    }
+                } else {
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+                        mixed[nt] = *reinterpret_cast<const f32x4*>(raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4);
+                }
+                bool ok[NT][4];
+                float tmax = TK_NEG_BIG;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = kt0 + nt * 16 + grp * 4 + i;
+                        ok[nt][i] = mine && page[nt] >= 0 && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
+                        if (ok[nt][i]) tmax = fmaxf(tmax, mixed[nt][i]);
+                    }
+                tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+                tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+                const float m_new = fmaxf(m_run[hh], tmax);
+                float psum = 0.f;
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float p = ok[nt][i] ? expf(mixed[nt][i] - m_new) : 0.f;
+                        mixed[nt][i] = p;
+                        psum += p;
+                    }
+                psum += __shfl_xor(psum, 16, WAVE);
+                psum += __shfl_xor(psum, 32, WAVE);
+                const float alpha = expf(m_run[hh] - m_new);
+                l_run[hh] = l_run[hh] * alpha + psum;
+                m_run[hh] = m_new;
+                Frag pf;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    pf.v[i] = from_f32<elem_t>(mixed[0][i]);
+                    pf.v[4 + i] = from_f32<elem_t>(NT > 1 ? mixed[NT - 1][i] : 0.f);
+                }
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[hh][dt][i] *= alpha;
+                    const int e = dt * 16 + r16;
+                    Frag vf = frag_zero();
+                    if (e < dv) {
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt) {
+                            const int pg = max(page[nt], 0), off = (kt0 + nt * 16) % ps + grp * 4;
+                            const elem_t* v0 = a.vpool + (((size_t)pg * KV + kvh) * dv + e) * ps + off;
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) vf.v[nt * 4 + i] = v0[i];
+                        }
+                    }
+                    mma_16x16x32(acc[hh][dt], vf, pf);
+                }
+            }
+            __syncthreads();
+        }
+    }
+    // O^T: lane holds value columns dt * 16 + grp * 4 + i of query r16
+    if (r0 + r16 < T) {
+#pragma unroll
+        for (int hh = 0; hh < HPW; ++hh) {
+            const int h = h0 + hh;
+            if (h >= H) break;
+            const float inv = 1.0f / l_run[hh];
+            elem_t* dst = a.out + ((size_t)(r0 + r16) * H + h) * dv;
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int e = dt * 16 + grp * 4 + i;
+                    if (e < dv) dst[e] = from_f32<elem_t>(acc[hh][dt][i] * inv);
+                }
+        }
+    }
+}
+
 }  // namespace ms
 
 using namespace ms;
@@ -261,4 +443,51 @@ extern "C" int ms_talking_attention(const void* q, const void* kpool, const void
                S, (elem_t*)out, H, KV, d, dv, ps, window, keep_first, scale};
     hipLaunchKernelGGL(talking_attention_kernel, dim3(T), dim3(256), lds, stream, a);
     return check_launch("attention");
+}
+
+// Whether the tile kernel takes these sizes (else the kernel of one row a block runs): head sizes that are multiples
+// of 8, at most 32 heads of at most 128 values, pages of a multiple of 16 positions.
+extern "C" int ms_talking_tile_takes(int H, int KV, int d, int dv, int ps) {
+    if (H < 1 || KV < 1 || H % KV || d % 8 || d > 256 || dv > 128 || dv < 1 || ps % 16 || H > 32) return 0;
+    const int nt = H <= 20 ? 2 : 1;
+    return ((size_t)H * 16 * nt * 16 + (size_t)H * H) * sizeof(float) <= (size_t)TK_MAX_LDS;
+}
+
+template <int HPW, int ND>
+static void launch_tile(const TalkArgs& a, const int* seq_q_len, int T, int NW, hipStream_t stream) {
+    const int nt = a.H <= 20 ? 2 : 1;
+    const size_t lds = ((size_t)a.H * 16 * nt * 16 + (size_t)a.H * a.H) * sizeof(float);
+    const dim3 grid(ceil_div(T, 16)), block(NW * 64);
+    if (nt == 2) hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 2>), grid, block, lds, stream, a, seq_q_len, T);
+    else hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 1>), grid, block, lds, stream, a, seq_q_len, T);
+}
+
+extern "C" int ms_talking_attention_tiles(const void* q, const void* kpool, const void* vpool, const float* talk, const int* block_table,
+                                          int table_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, int S,
+                                          void* out, int T, int H, int KV, int d, int dv, int ps, int window, int keep_first, float scale,
+                                          hipStream_t stream) {
+    MS_REQUIRE(T > 0 && S > 0, "attention: empty problem");
+    MS_REQUIRE(ms_talking_tile_takes(H, KV, d, dv, ps), "attention in tiles: %d heads over %d, keys of %d, values of %d, pages of %d are not taken",
+               H, KV, d, dv, ps);
+    MS_REQUIRE(window >= 0 && keep_first >= 0, "attention: window %d, %d first tokens kept", window, keep_first);
+    MS_REQUIRE(q && kpool && vpool && block_table && seq_q_start && seq_q_len && seq_pos0 && out, "attention: a buffer is missing");
+    MS_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kpool) | reinterpret_cast<uintptr_t>(vpool)) & 15) == 0,
+               "attention in tiles: operands must be 16-byte aligned");
+    TalkArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, talk, block_table, table_stride, seq_q_start, seq_pos0,
+               S, (elem_t*)out, H, KV, d, dv, ps, window, keep_first, scale};
+    const int hpw = H <= 8 ? 1 : H <= 16 ? 2 : 4, nw = ceil_div(H, hpw), nd = ceil_div(dv, 16);
+#define MS_TILE(HP, NDD) launch_tile<HP, NDD>(a, seq_q_len, T, nw, stream)
+#define MS_TILE_ND(HP)                      \
+    do {                                    \
+        if (nd <= 1) MS_TILE(HP, 1);        \
+        else if (nd <= 2) MS_TILE(HP, 2);   \
+        else if (nd <= 4) MS_TILE(HP, 4);   \
+        else MS_TILE(HP, 8);                \
+    } while (0)
+    if (hpw == 1) MS_TILE_ND(1);
+    else if (hpw == 2) MS_TILE_ND(2);
+    else MS_TILE_ND(4);
+#undef MS_TILE_ND
+#undef MS_TILE
+    return check_launch("attention in tiles");
 }

@@ -699,12 +699,20 @@ class HipOps:
             _c_int(H), _c_int(KV), _c_int(d), _c_int(dv), _c_int(page_size), self._stream()))
         return q, v_raw
 
+    TILE_MIN_ROWS = 8  # a step of at least this many rows that is not plain decoding runs in tiles of 16 rows
+
+    def talking_tile_takes(self, H: int, KV: int, d: int, dv: int, page_size: int) -> bool:
+        """Whether the kernel that takes 16 rows a block on the matrix cores is built for these sizes."""
+        return bool(self._plan("ms_talking_tile_takes", H, KV, d, dv, page_size, lib=self._extra_lib("talking")))
+
     def talking_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, talk: Optional[torch.Tensor],
                           block_table: torch.Tensor, seq_q_start: torch.Tensor, seq_pos0: torch.Tensor, H: int, KV: int, d: int, dv: int,
-                          page_size: int, window: Optional[int], keep_first: int, scale: float) -> torch.Tensor:
+                          page_size: int, window: Optional[int], keep_first: int, scale: float,
+                          seq_q_len: Optional[torch.Tensor] = None, tiles: bool = False) -> torch.Tensor:
         """Attention of every row over the keys it sees: the last ``window`` positions up to its own (None: all) and
         the request's first ``keep_first``.  ``talk`` float32 ``[H, H]`` mixes the heads' scaled scores before the
-        softmax (None: no exchange).  Returns ``[T, H * dv]`` in the element type."""
+        softmax (None: no exchange).  Returns ``[T, H * dv]`` in the element type.  ``tiles`` (with ``seq_q_len``): 16
+        rows a block on the matrix cores, for steps of many rows; else one row a block, for decoding."""
         lib = self._extra_lib("talking")
         T = q.shape[0]
         self._want(q, self.dtype, "attention q", T, H * d)
@@ -720,6 +728,13 @@ class HipOps:
         self._want(seq_q_start, torch.int32, "seq_q_start", S)
         self._want(seq_pos0, torch.int32, "seq_pos0", S)
         out = torch.empty((T, H * dv), dtype=self.dtype, device=q.device)
+        if tiles and self.talking_tile_takes(H, KV, d, dv, page_size):
+            self._want(seq_q_len, torch.int32, "seq_q_len", S)
+            self._check(lib, lib.ms_talking_attention_tiles(
+                _ptr(q), _ptr(kpool), _ptr(vpool), _ptr(talk), _ptr(block_table), _c_int(block_table.shape[1]), _ptr(seq_q_start),
+                _ptr(seq_q_len), _ptr(seq_pos0), _c_int(S), _ptr(out), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv),
+                _c_int(page_size), _c_int(window or 0), _c_int(keep_first), _c_float(scale), self._stream()))
+            return out
         self._check(lib, lib.ms_talking_attention(
             _ptr(q), _ptr(kpool), _ptr(vpool), _ptr(talk), _ptr(block_table), _c_int(block_table.shape[1]), _ptr(seq_q_start),
             _ptr(seq_pos0), _c_int(S), _ptr(out), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv), _c_int(page_size),

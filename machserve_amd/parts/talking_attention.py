@@ -87,6 +87,9 @@ class TalkingAttention(Mixer):
                                      view.page_size)
         if s.value_blend == "source":
             ctx.shared[shared] = own
+        # a step of many rows runs in tiles of 16 rows on the matrix cores, single decoded rows one row a block
+        tiles = not ctx.decode_only and ctx.n_rows >= getattr(ops, "TILE_MIN_ROWS", 1 << 30)
         o = ops.talking_attention(q, self.kpool, self.vpool, self.talk, view.block_table, ctx.seq_q_start, ctx.seq_pos0, s.heads,
-                                  s.kv_heads, s.head_dim, s.v_head_dim, view.page_size, s.window, s.keep_first, float(s.scale))
+                                  s.kv_heads, s.head_dim, s.v_head_dim, view.page_size, s.window, s.keep_first, float(s.scale),
+                                  ctx.seq_q_len, tiles)
         stream.add_linear(o, self.w_o)

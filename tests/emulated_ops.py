@@ -285,7 +285,7 @@ class EmulatedOps:
         return q, own
 
     def talking_attention(self, q, kpool, vpool, talk, block_table, seq_q_start, seq_pos0, H, KV, d, dv, page_size, window,
-                          keep_first, scale):
+                          keep_first, scale, seq_q_len=None, tiles=False):
         T, S = q.shape[0], seq_q_start.numel()
         rep = H // KV
         out = torch.zeros(T, H, dv)

@@ -36,7 +36,7 @@ def i32(values):
 
 def close(got, want, dtype, what="", scale_by=None):
     got, want = got.float().cpu().double(), want.double().cpu()
-    bound = (1e-5 if dtype == torch.float32 else 2e-2) * float((scale_by if scale_by is not None else want).abs().max()) + 1e-6
+    bound = (4e-5 if dtype == torch.float32 else 2e-2) * float((scale_by if scale_by is not None else want).abs().max()) + 1e-6
     err = float((got - want).abs().max())
     assert err <= bound, f"{what}: error {err:.3e} over {bound:.3e}"
 
@@ -147,7 +147,7 @@ def test_lightning_attention_in_one_step_and_in_many(dtype, H, d, dv):
     close(gated, P.rms(o.double().cpu(), 1e-5) * w.double() * torch.sigmoid(rows[:, 2 * H * d + H * dv:].double()), dtype, "gated norm")
 
 
-def _attention_case(dtype, H, KV, d, dv, ps, lens_before, lens_now, window, keep, rot, talk, seed, spike=None, normed=True):
+def _attention_case(dtype, H, KV, d, dv, ps, lens_before, lens_now, window, keep, rot, talk, seed, spike=None, normed=True, tiles=False):
     """Requests with `lens_before` tokens in the cache bring `lens_now` more.  Everything goes through the two kernels,
     step by step, and is compared with the plain attention over each whole request.  `spike = (request, key position)`
     makes that key's score with every query huge (the rows are then neither normed nor rotated, which would undo it)."""
@@ -190,7 +190,7 @@ def _attention_case(dtype, H, KV, d, dv, ps, lens_before, lens_now, window, keep
         q, _ = ops.talking_prepare(dev(rows).unsqueeze(0), dev(qn) if normed else None, dev(kn) if normed else None, 1e-5, dev(positions.int()), dev(inv) if rot else None, rot, factor,
                                    None, None, False, dev(slot_map.int()), kpool, vpool, H, KV, d, dv, ps)
         out = ops.talking_attention(q, kpool, vpool, dev(T_) if talk else None, dev(table[live]), i32(q_start), i32([start[s] for s in live]),
-                                    H, KV, d, dv, ps, window, keep, scale)
+                                    H, KV, d, dv, ps, window, keep, scale, i32([lens[s] for s in live]), tiles)
         if phase == "now":
             for i, s in enumerate(live):
                 got[s] = out[q_start[i]:q_start[i] + lens[s]].float().cpu()
@@ -221,15 +221,19 @@ def _attention_case(dtype, H, KV, d, dv, ps, lens_before, lens_now, window, keep
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,KV,d,dv,rot", [(4, 2, 32, 16, 16), (6, 1, 24, 40, 24), (3, 3, 8, 8, 0), (8, 8, 64, 64, 32), (5, 1, 20, 12, 4)])
-def test_talking_attention_kernels(dtype, H, KV, d, dv, rot):
+@pytest.mark.parametrize("tiles", [False, True])
+@pytest.mark.parametrize("H,KV,d,dv,rot", [(4, 2, 32, 16, 16), (6, 1, 24, 40, 24), (3, 3, 8, 8, 0), (8, 8, 64, 64, 32), (5, 1, 20, 12, 4),
+                                           (12, 4, 48, 80, 48), (24, 3, 16, 128, 8), (32, 32, 40, 16, 40)])
+def test_talking_attention_kernels(dtype, H, KV, d, dv, rot, tiles):
+    """One row a block, and 16 rows a block on the matrix cores (sizes that kernel does not take run in the other)."""
     # prompts, portions of prompts that go on, and single decoded rows side by side; a window that crosses pages
-    _attention_case(dtype, H, KV, d, dv, 16, [0, 40, 70, 5], [50, 13, 1, 1], 24, 3, rot, True, seed=H)
-    _attention_case(dtype, H, KV, d, dv, 16, [0, 31], [130, 1], None, 0, rot, H % 2 == 0, seed=H + 1)    # all keys, far ones too
+    _attention_case(dtype, H, KV, d, dv, 16, [0, 40, 70, 5], [50, 13, 1, 1], 24, 3, rot, True, seed=H, tiles=tiles)
+    _attention_case(dtype, H, KV, d, dv, 16, [0, 31], [130, 1], None, 0, rot, H % 2 == 0, seed=H + 1, tiles=tiles)    # all keys, far ones too
+    _attention_case(dtype, H, KV, d, dv, 32, [3, 0, 100], [7, 9, 21], 40, 35, rot, True, seed=H + 2, tiles=tiles)   # kept tokens beyond a page
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("decoded", [False, True])
+@pytest.mark.parametrize("decoded", [False, True, "tiles"])
 @pytest.mark.parametrize("edge", ["inside the window", "outside the window", "kept", "not kept", "page border", "own"])
 def test_a_key_that_stands_out_shows_at_every_edge(dtype, decoded, edge):
     """One key's score is made huge: its value is the output if the row sees it, and absent if not, so a window or
@@ -237,8 +241,9 @@ def test_a_key_that_stands_out_shows_at_every_edge(dtype, decoded, edge):
     window, keep, ps, n = 20, 5, 16, 64
     key = {"inside the window": n - window, "outside the window": n - window - 1, "kept": keep - 1, "not kept": keep,
            "page border": 48, "own": n - 1}[edge]
-    before, now = ([n - 1], [1]) if decoded else ([0], [n])
-    got = _attention_case(dtype, 4, 2, 16, 16, ps, before, now, window, keep, 0, True, seed=11, spike=(0, key), normed=False)
+    before, now = ([n - 1], [1]) if decoded is True else ([0], [n])
+    got = _attention_case(dtype, 4, 2, 16, 16, ps, before, now, window, keep, 0, True, seed=11, spike=(0, key), normed=False,
+                          tiles=decoded == "tiles")
     assert len(got) == 1
 
 
