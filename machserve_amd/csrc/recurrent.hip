@@ -66,15 +66,30 @@ __global__ __launch_bounds__(256) void conv_state_kernel(const elem_t* __restric
 }
 
 // ---- step sizes ------------------------------------------------------------------------
-// dt[t, c] = softplus(b[c] + sum_r w[c, r] * low[t, r]), low = the first R columns of the rows of `dbc`
-__global__ __launch_bounds__(256) void dt_softplus_kernel(const float* __restrict__ dbc, int ldb, const float* __restrict__ w,
-                                                          const float* __restrict__ b, float* __restrict__ dt, int C, int R) {
-    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+// dt[t, c] = softplus(b[c] + sum_r wt[r, c] * low[t, r]), low = the first R columns of the rows of `dbc`; `wt` is the
+// projection transposed, [R, C], so that the threads of a wave read neighbouring numbers.  A block takes DT_ROWS rows
+// and 256 channels: a weight is read once for all of its rows.
+constexpr int DT_ROWS = 8;
+__global__ __launch_bounds__(256) void dt_softplus_kernel(const float* __restrict__ dbc, int ldb, const float* __restrict__ wt,
+                                                          const float* __restrict__ b, float* __restrict__ dt, int T, int C, int R) {
+    extern __shared__ float low[];  // [DT_ROWS][R]
+    const int t0 = blockIdx.x * DT_ROWS, c = blockIdx.y * 256 + threadIdx.x;
+    const int nr = min(DT_ROWS, T - t0);
+    for (int i = threadIdx.x; i < nr * R; i += 256) low[i] = dbc[(size_t)(t0 + i / R) * ldb + i % R];
+    __syncthreads();
     if (c >= C) return;
-    const float* low = dbc + (size_t)t * ldb;
-    float acc = b ? b[c] : 0.f;
-    for (int r = 0; r < R; ++r) acc += w[(size_t)c * R + r] * low[r];
-    dt[(size_t)t * C + c] = softplus_f(acc);
+    float acc[DT_ROWS];
+    const float bias = b ? b[c] : 0.f;
+#pragma unroll
+    for (int k = 0; k < DT_ROWS; ++k) acc[k] = bias;
+    for (int r = 0; r < R; ++r) {
+        const float w = wt[(size_t)r * C + c];
+#pragma unroll
+        for (int k = 0; k < DT_ROWS; ++k) acc[k] += w * low[(k < nr ? k : 0) * R + r];
+    }
+#pragma unroll
+    for (int k = 0; k < DT_ROWS; ++k)
+        if (k < nr) dt[(size_t)(t0 + k) * C + c] = softplus_f(acc[k]);
 }
 
 // ---- selective scan --------------------------------------------------------------------
@@ -170,6 +185,174 @@ __global__ __launch_bounds__(64) void lightning_kernel(const elem_t* __restrict_
     }
 }
 
+// ---- the same in chunks of 32 tokens on the matrix cores --------------------------------------
+// For a chunk with tokens i, j = 0 .. n - 1 and the state S before it:
+//   o_i = decay^(i + 1) S^T q_i + sum_{j <= i} decay^(i - j) (q_i . k_j) v_j,      S <- decay^n S + sum_j decay^(n - 1 - j) k_j v_j^T,
+// which equals the recurrence token after token.  A block is one (request, head) and walks the request's chunks in
+// order; wave w owns the value columns of the 16-wide tiles w, w + 4, ... and keeps its part of S in 32-bit
+// accumulators throughout.  q, k and v are activated in 32-bit and rounded to the element type as operands of the
+// products; the scores times their decays, and the state, are rounded only as operands (not at all in the 32-bit
+// build), and every sum is 32-bit.
+constexpr int LC = 32;  // tokens of a chunk
+template <int DT, int CT>
+__global__ __launch_bounds__(256) void lightning_chunk_kernel(const elem_t* __restrict__ qkv, int ld, int col_q, int col_k, int col_v,
+                                                              const float* __restrict__ decay, float* __restrict__ state,
+                                                              const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
+                                                              const int* __restrict__ seq_slot, float* __restrict__ o, int H, int d, int dv) {
+    constexpr int DP = DT * 16, VP = CT * 64;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    elem_t* Qs = reinterpret_cast<elem_t*>(smem);  // [LC][DP]
+    elem_t* Ks = Qs + LC * DP;                     // [LC][DP]
+    elem_t* VT = Ks + LC * DP;                     // [VP][LC]: values transposed
+    elem_t* Ps = VT + VP * LC;                     // [LC][LC]: scores times decays
+    float* pw = reinterpret_cast<float*>(Ps + LC * LC);  // [LC + 1]: decay^k
+    const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r16 = lane & 15, grp = lane >> 4;
+    const int q0 = seq_q_start[s], n_rows = seq_q_len[s];
+    float* st = state + (((size_t)seq_slot[s] * H + h) * d) * dv;
+    const float lam = decay[h];
+    if (tid <= LC) pw[tid] = powf(lam, (float)tid);
+    f32x4 S[DT][CT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+            const int e = (wave + 4 * c) * 16 + r16;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int dd = dt * 16 + grp * 4 + i;
+                S[dt][c][i] = (dd < d && e < dv) ? st[(size_t)dd * dv + e] : 0.f;
+            }
+        }
+    const size_t orow = (size_t)H * dv;
+    for (int i0 = 0; i0 < n_rows; i0 += LC) {
+        const int n = min(LC, n_rows - i0);
+        __syncthreads();  // the chunk before has been read
+        for (int idx = tid; idx < LC * DP; idx += 256) {
+            const int r = idx / DP, c = idx - r * DP;
+            float qv = 0.f, kv = 0.f;
+            if (r < n && c < d) {
+                const elem_t* row = qkv + (size_t)(q0 + i0 + r) * ld + h * d + c;
+                qv = silu_f(to_f32(row[col_q]));
+                kv = silu_f(to_f32(row[col_k]));
+            }
+            Qs[idx] = from_f32<elem_t>(qv);
+            Ks[idx] = from_f32<elem_t>(kv);
+        }
+        for (int idx = tid; idx < LC * VP; idx += 256) {
+            const int r = idx / VP, e = idx - r * VP;
+            float v = 0.f;
+            if (r < n && e < dv) v = silu_f(to_f32(qkv[(size_t)(q0 + i0 + r) * ld + col_v + h * dv + e]));
+            VT[e * LC + r] = from_f32<elem_t>(v);
+        }
+        __syncthreads();
+        {   // a quarter of the scores a wave: rows rt, columns ct
+            const int rt = wave >> 1, ct = wave & 1;
+            f32x4 p = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < DT / 2; ++ks) {
+                const Frag qa = frag_load(&Qs[(rt * 16 + r16) * DP + ks * 32 + grp * 8]);
+                const Frag kb = frag_load(&Ks[(ct * 16 + r16) * DP + ks * 32 + grp * 8]);
+                mma_16x16x32(p, qa, kb);
+            }
+            const int j = ct * 16 + r16;
+#pragma unroll
+            for (int ii = 0; ii < 4; ++ii) {
+                const int i = rt * 16 + grp * 4 + ii;
+                Ps[i * LC + j] = from_f32<elem_t>(j <= i ? p[ii] * pw[i - j] : 0.f);
+            }
+        }
+        // what the state before the chunk gives: rows are tokens, the sum runs over the head's numbers in pairs of tiles
+        f32x4 O[2][CT];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+            for (int c = 0; c < CT; ++c) O[rt][c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t2 = 0; t2 < DT / 2; ++t2) {
+            Frag qa[2];
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                const elem_t* qp = &Qs[(rt * 16 + r16) * DP + t2 * 32 + grp * 4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    qa[rt].v[i] = qp[i];
+                    qa[rt].v[4 + i] = qp[16 + i];
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < CT; ++c) {
+                Frag sb;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    sb.v[i] = from_f32<elem_t>(S[2 * t2][c][i]);
+                    sb.v[4 + i] = from_f32<elem_t>(S[2 * t2 + 1][c][i]);
+                }
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt) mma_16x16x32(O[rt][c], qa[rt], sb);
+            }
+        }
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+            for (int ii = 0; ii < 4; ++ii) {
+                const float f = pw[rt * 16 + grp * 4 + ii + 1];
+#pragma unroll
+                for (int c = 0; c < CT; ++c) O[rt][c][ii] *= f;
+            }
+        __syncthreads();  // the scores are complete
+        Frag vb[CT];
+#pragma unroll
+        for (int c = 0; c < CT; ++c) vb[c] = frag_load(&VT[((wave + 4 * c) * 16 + r16) * LC + grp * 8]);
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            const Frag pa = frag_load(&Ps[(rt * 16 + r16) * LC + grp * 8]);
+#pragma unroll
+            for (int c = 0; c < CT; ++c) mma_16x16x32(O[rt][c], pa, vb[c]);
+        }
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+            for (int c = 0; c < CT; ++c) {
+                const int e = (wave + 4 * c) * 16 + r16;
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii) {
+                    const int i = rt * 16 + grp * 4 + ii;
+                    if (i < n && e < dv) o[(size_t)(q0 + i0 + i) * orow + (size_t)h * dv + e] = O[rt][c][ii];
+                }
+            }
+        // the state after the chunk
+        const float ln = pw[n];
+        float kw[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int j = grp * 8 + i;
+            kw[i] = j < n ? pw[n - 1 - j] : 0.f;
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            Frag ka;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ka.v[i] = from_f32<elem_t>(to_f32(Ks[(grp * 8 + i) * DP + dt * 16 + r16]) * kw[i]);
+#pragma unroll
+            for (int c = 0; c < CT; ++c) {
+                S[dt][c] *= ln;
+                mma_16x16x32(S[dt][c], ka, vb[c]);
+            }
+        }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+            const int e = (wave + 4 * c) * 16 + r16;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int dd = dt * 16 + grp * 4 + i;
+                if (dd < d && e < dv) st[(size_t)dd * dv + e] = S[dt][c][i];
+            }
+        }
+}
+
 // out[t, :] = o[t, :] / sqrt(mean(o[t, :]^2) + eps) * w * sigmoid(gate[t, :])
 __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const float* __restrict__ o, const elem_t* __restrict__ gate, int ldg,
                                                             const float* __restrict__ w, elem_t* __restrict__ out, int n, float eps) {
@@ -211,11 +394,14 @@ extern "C" int ms_causal_conv(const void* x, int ld, const float* w, const float
     return 0;
 }
 
+// w: the projection of the step sizes transposed, [R, C]
 extern "C" int ms_dt_softplus(const float* dbc, int ldb, const float* w, const float* b, float* dt, int T, int C, int R,
                               hipStream_t stream) {
     MS_REQUIRE(T > 0 && C > 0 && R > 0 && ldb >= R, "step sizes: T=%d C=%d R=%d ld=%d", T, C, R, ldb);
     MS_REQUIRE(dbc && w && dt, "step sizes: a buffer is missing");
-    hipLaunchKernelGGL(dt_softplus_kernel, dim3(T, ceil_div(C, 256)), dim3(256), 0, stream, dbc, ldb, w, b, dt, C, R);
+    MS_REQUIRE((size_t)DT_ROWS * R * sizeof(float) <= 48 * 1024, "step sizes: a bottleneck of %d is too wide", R);
+    hipLaunchKernelGGL(dt_softplus_kernel, dim3(ceil_div(T, DT_ROWS), ceil_div(C, 256)), dim3(256), (size_t)DT_ROWS * R * sizeof(float), stream,
+                       dbc, ldb, w, b, dt, T, C, R);
     return check_launch("step sizes");
 }
 
@@ -265,4 +451,31 @@ extern "C" int ms_gated_rmsnorm(const float* o, const void* gate, int ldg, const
     MS_REQUIRE(o && gate && w && out, "gated norm: a buffer is missing");
     hipLaunchKernelGGL(gated_rmsnorm_kernel, dim3(T), dim3(256), 0, stream, o, (const elem_t*)gate, ldg, w, (elem_t*)out, n, eps);
     return check_launch("gated norm");
+}
+
+// Whether the kernel that walks a request in chunks on the matrix cores takes these head sizes.
+extern "C" int ms_lightning_chunked_takes(int d, int dv) { return d >= 1 && d <= 128 && dv >= 1 && dv <= 128; }
+
+extern "C" int ms_lightning_chunked(const void* qkv, int ld, int col_q, int col_k, int col_v, const float* decay, float* state,
+                                    const int* seq_q_start, const int* seq_q_len, const int* seq_slot, int S, float* o, int T, int H,
+                                    int d, int dv, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && S > 0 && H > 0, "lightning attention: T=%d S=%d H=%d", T, S, H);
+    MS_REQUIRE(ms_lightning_chunked_takes(d, dv), "lightning attention in chunks: heads of %d and values of %d are not taken", d, dv);
+    MS_REQUIRE(col_q >= 0 && col_k >= 0 && col_v >= 0 && col_q + H * d <= ld && col_k + H * d <= ld && col_v + H * dv <= ld,
+               "lightning attention: columns %d, %d, %d of rows of %d", col_q, col_k, col_v, ld);
+    MS_REQUIRE(qkv && decay && state && seq_q_start && seq_q_len && seq_slot && o, "lightning attention: a buffer is missing");
+    const dim3 grid(S, H);
+    const int dtl = d <= 32 ? 2 : d <= 64 ? 4 : 8, ctl = dv <= 64 ? 1 : 2;
+#define MS_LCH(DTT, CTT)                                                                                                            \
+    hipLaunchKernelGGL((lightning_chunk_kernel<DTT, CTT>), grid, dim3(256),                                                          \
+                       sizeof(elem_t) * (2 * LC * DTT * 16 + CTT * 64 * LC + LC * LC) + sizeof(float) * (LC + 1 + 3), stream,       \
+                       (const elem_t*)qkv, ld, col_q, col_k, col_v, decay, state, seq_q_start, seq_q_len, seq_slot, o, H, d, dv)
+    if (dtl == 2 && ctl == 1) MS_LCH(2, 1);
+    else if (dtl == 2) MS_LCH(2, 2);
+    else if (dtl == 4 && ctl == 1) MS_LCH(4, 1);
+    else if (dtl == 4) MS_LCH(4, 2);
+    else if (ctl == 1) MS_LCH(8, 1);
+    else MS_LCH(8, 2);
+#undef MS_LCH
+    return check_launch("lightning attention in chunks");
 }

@@ -598,14 +598,14 @@ class HipOps:
                        seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor) -> torch.Tensor:
         """The scan of a Mamba layer over the step's rows.  ``x [T, C]``: the convolved input; ``xz [T, 2 C]``: its second
         half is the gate; ``dbc`` float32 ``[T, dt_rank + 2 n_states]``: step size input, B and C.  Step sizes are
-        ``softplus(w_dt @ low + b_dt)``; ``state`` float32 ``[slots, C, n_states]`` is carried on.  Returns
+        ``softplus(low @ w_dt + b_dt)`` with ``w_dt [dt_rank, C]``, the projection transposed; ``state`` float32 ``[slots, C, n_states]`` is carried on.  Returns
         ``y * silu(gate)`` ``[T, C]``."""
         lib = self._extra_lib("recurrent")
         T, C = x.shape
         self._want(x, self.dtype, "scan input")
         self._want(xz, self.dtype, "scan gate", T, 2 * C)
         self._want(dbc, torch.float32, "scan step input", T, dt_rank + 2 * n_states)
-        self._want(w_dt, torch.float32, "scan step weight", C, dt_rank)
+        self._want(w_dt, torch.float32, "scan step weight (transposed)", dt_rank, C)
         if b_dt is not None:
             self._want(b_dt, torch.float32, "scan step bias", C)
         self._want(a_log, torch.float32, "scan A_log", C, n_states)
@@ -626,10 +626,11 @@ class HipOps:
         return y
 
     def lightning_attention(self, qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.Tensor, state: torch.Tensor,
-                            seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor) -> torch.Tensor:
+                            seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor, chunked: bool = False) -> torch.Tensor:
         """Linear attention with a decay per head over the step's rows.  ``qkvg [T, ld]`` holds q ``[heads, dim]``, k
         ``[heads, dim]``, v ``[heads, vdim]`` (and whatever follows) before their SiLU; ``state`` float32
-        ``[slots, heads, dim, vdim]`` is carried on.  Returns float32 ``[T, heads * vdim]``."""
+        ``[slots, heads, dim, vdim]`` is carried on.  Returns float32 ``[T, heads * vdim]``.  ``chunked``: a request's rows
+        in chunks of 32 on the matrix cores (steps of many rows), else token after token (decoding)."""
         lib = self._extra_lib("recurrent")
         T, ld = qkvg.shape
         self._want(qkvg, self.dtype, "lightning q/k/v")
@@ -637,7 +638,8 @@ class HipOps:
         self._want(state, torch.float32, "lightning state", state.shape[0], heads, dim, vdim)
         S = self._seq_operands("lightning", seq_q_start, seq_q_len, seq_slot)
         o = torch.empty((T, heads * vdim), dtype=torch.float32, device=qkvg.device)
-        self._check(lib, lib.ms_lightning(_ptr(qkvg), _c_int(ld), _c_int(0), _c_int(heads * dim), _c_int(2 * heads * dim), _ptr(decay),
+        fn = lib.ms_lightning_chunked if chunked and self._plan("ms_lightning_chunked_takes", dim, vdim, lib=lib) else lib.ms_lightning
+        self._check(lib, fn(_ptr(qkvg), _c_int(ld), _c_int(0), _c_int(heads * dim), _c_int(2 * heads * dim), _ptr(decay),
                                           _ptr(state), _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(o),
                                           _c_int(T), _c_int(heads), _c_int(dim), _c_int(vdim), self._stream()))
         return o

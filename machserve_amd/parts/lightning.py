@@ -50,7 +50,8 @@ class LightningAttention(Mixer):
     def forward(self, h, stream, ctx):
         s, ops = self.spec, self.rt.ops
         qkvg = ops.linear(h, self.w_qkvg)
+        # single decoded rows go token after token; portions of prompts in chunks on the matrix cores
         o = ops.lightning_attention(qkvg, s.heads, s.head_dim, s.v_head_dim, self.decay, self.state["kv"], ctx.seq_q_start,
-                                    ctx.seq_q_len, ctx.seq_slot)
+                                    ctx.seq_q_len, ctx.seq_slot, not ctx.decode_only)
         y = ops.gated_rmsnorm(o, qkvg, 2 * self.nqk + self.nv, self.norm_w, s.norm_eps)
         stream.add_linear(y, self.w_o)

@@ -38,7 +38,9 @@ class SelectiveScan(Mixer):
     def load(self, t):
         self.w_in, self.w_x, self.w_o = t["in.weight"], t["x.weight"], t["o.weight"]
         self.conv_w, self.conv_b = t["conv.weight"], t["conv.bias"]
-        self.w_dt, self.b_dt, self.a_log, self.d_skip = t["dt.weight"], t["dt.bias"], t["A_log"], t["D"]
+        # the step sizes' projection is kept transposed, [dt_rank, channels]: the kernel's threads are channels
+        self.w_dt = t["dt.weight"].t().contiguous()
+        self.b_dt, self.a_log, self.d_skip = t["dt.bias"], t["A_log"], t["D"]
 
     def cache_request(self):
         s = self.spec

@@ -215,7 +215,7 @@ class EmulatedOps:
     def selective_scan(self, x, xz, dbc, dt_rank, n_states, w_dt, b_dt, a_log, d_skip, state, seq_q_start, seq_q_len, seq_slot):
         T, C = x.shape
         low, B, Cm = dbc[:, :dt_rank], dbc[:, dt_rank:dt_rank + n_states], dbc[:, dt_rank + n_states:]
-        dt = torch.nn.functional.softplus(low @ w_dt.t() + (0 if b_dt is None else b_dt))
+        dt = torch.nn.functional.softplus(low @ w_dt + (0 if b_dt is None else b_dt))   # w_dt comes transposed, [dt_rank, C]
         A = -torch.exp(a_log)
         xf, z = x.float(), xz[:, C:].float()
         y = torch.empty(T, C)
@@ -227,7 +227,7 @@ class EmulatedOps:
             state[slot] = S
         return self._r(y * _act(z, "silu"))
 
-    def lightning_attention(self, qkvg, heads, dim, vdim, decay, state, seq_q_start, seq_q_len, seq_slot):
+    def lightning_attention(self, qkvg, heads, dim, vdim, decay, state, seq_q_start, seq_q_len, seq_slot, chunked=False):
         T = qkvg.shape[0]
         f = qkvg.float()
         q = _act(f[:, :heads * dim], "silu").view(T, heads, dim)

@@ -108,7 +108,7 @@ def test_selective_scan_in_one_step_and_in_many(dtype, C, N, R):
         state[0] = 7.0   # another request's: must stay
         got, at = [], 0
         for c in cuts:
-            got.append(ops.selective_scan(dev(x[at:at + c], dtype), dev(xz[at:at + c], dtype), dev(dbc[at:at + c]), R, N, dev(w_dt),
+            got.append(ops.selective_scan(dev(x[at:at + c], dtype), dev(xz[at:at + c], dtype), dev(dbc[at:at + c]), R, N, dev(w_dt.t()),
                                           dev(b_dt), dev(a_log), dev(dsk), state, i32([0]), i32([c]), i32([1])))
             at += c
         close(torch.cat(got), want, dtype, f"scan cut as {cuts[:4]}")
@@ -117,11 +117,13 @@ def test_selective_scan_in_one_step_and_in_many(dtype, C, N, R):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,d,dv", [(2, 16, 24), (1, 40, 8), (3, 8, 70), (2, 72, 16)])
-def test_lightning_attention_in_one_step_and_in_many(dtype, H, d, dv):
+@pytest.mark.parametrize("chunked", [False, True])
+@pytest.mark.parametrize("H,d,dv", [(2, 16, 24), (1, 40, 8), (3, 8, 70), (2, 72, 16), (2, 128, 128), (1, 136, 8)])
+def test_lightning_attention_in_one_step_and_in_many(dtype, H, d, dv, chunked):
+    """Token after token, and in chunks on the matrix cores (head sizes that kernel does not take run in the other)."""
     ops = ops_of(dtype)
     torch.manual_seed(d)
-    n = 45
+    n = 77
     ld = 2 * H * d + 2 * H * dv
     rows = torch.randn(n, ld).to(dtype).float()
     decay = torch.tensor([0.6, 0.95, 0.999][:H])
@@ -133,14 +135,15 @@ def test_lightning_attention_in_one_step_and_in_many(dtype, H, d, dv):
         S = decay.double()[:, None, None] * S + k[i][:, :, None] * v[i][:, None, :]
         want[i] = torch.einsum("hde,hd->he", S, q[i])
     want = want.reshape(n, H * dv)
-    for cuts in ([n], [1] * n, [16, 17, 2, 10]):
+    for cuts in ([n], [1] * n, [16, 17, 2, 32, 10]):
         state = torch.zeros(2, H, d, dv, device=DEV)
         got, at = [], 0
         for c in cuts:
-            got.append(ops.lightning_attention(dev(rows[at:at + c], dtype), H, d, dv, dev(decay), state, i32([0]), i32([c]), i32([1])))
+            got.append(ops.lightning_attention(dev(rows[at:at + c], dtype), H, d, dv, dev(decay), state, i32([0]), i32([c]), i32([1]), chunked))
             at += c
-        close(torch.cat(got), want, torch.float32, f"lightning cut as {cuts[:4]}")
-        close(state[1], S, torch.float32, "the state after the last token")
+        # in chunks the activations, the decayed scores and the state are rounded to the element type as operands
+        close(torch.cat(got), want, dtype if chunked else torch.float32, f"lightning cut as {cuts[:4]}")
+        close(state[1], S, dtype if chunked else torch.float32, "the state after the last token")
     w = torch.randn(H * dv)
     o = torch.cat(got)
     gated = ops.gated_rmsnorm(o, dev(rows, dtype), 2 * H * d + H * dv, dev(w), 1e-5)
