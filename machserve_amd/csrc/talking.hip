@@ -403,6 +403,179 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
     }
 }
 
+// ---- one row a block, its keys cut over several blocks ------------------------------------------
+// For decoding: block (t, y) takes the y-th share of the 64-position tiles that row t sees, with 16-byte loads of keys
+// and values, and leaves a running maximum, sum and unnormalised output per head; a second kernel merges the shares
+// (one share: the block normalises and writes the output itself).  Needs head sizes that are multiples of 8 and pages
+// of a multiple of 16 positions.
+constexpr int TK_MAX_REP = 16;
+
+__device__ __forceinline__ void load8(const elem_t* p, float* out) {
+    const Frag f = frag_load(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = to_f32(f.v[i]);
+}
+
+__global__ __launch_bounds__(256) void talking_attention_split_kernel(TalkArgs a, int n_split, float* __restrict__ part_o,
+                                                                      float* __restrict__ part_ml) {
+    extern __shared__ float lds[];
+    const int H = a.H, d = a.d, dv = a.dv, KV = a.KV, rep = H / KV, ps = a.ps;
+    float* qs = lds;                      // [H * d], scaled
+    float* raw = qs + H * d;              // [H][64]
+    float* mix = raw + H * TK_KEYS;       // [H][64]: mixed scores, then weights
+    float* head_m = mix + H * TK_KEYS;
+    float* head_l = head_m + H;
+    float* head_a = head_l + H;
+    int* page_of = reinterpret_cast<int*>(head_a + H);  // [4] pages of the tile's 16-position parts, -1: none
+    const int t = blockIdx.x, y = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int s = seq_of_row(t, a.seq_q_start, a.S);
+    const int pos = a.seq_pos0[s] + (t - a.seq_q_start[s]);
+    const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+    const int n_first = min(a.keep_first, lo);
+    const int a_end = (n_first + TK_KEYS - 1) / TK_KEYS;
+    const int b_begin = max(a_end, lo / TK_KEYS), b_end = pos / TK_KEYS + 1;
+    const int n_tiles = a_end + (b_end - b_begin);
+    const int per = (n_tiles + n_split - 1) / n_split;
+    const int it0 = y * per, it1 = min(n_tiles, it0 + per);
+    const int* table = a.block_table + (size_t)s * a.table_stride;
+    for (int c = tid; c < H * d; c += 256) qs[c] = to_f32(a.q[(size_t)t * H * d + c]) * a.scale;
+    for (int h = tid; h < H; h += 256) {
+        head_m[h] = -INFINITY;
+        head_l[h] = 0.f;
+    }
+    float acc[TK_MAX_OUT];
+#pragma unroll
+    for (int i = 0; i < TK_MAX_OUT; ++i) acc[i] = 0.f;
+    const int n_out = H * dv;
+    for (int it = it0; it < it1; ++it) {
+        const int kt0 = (it < a_end ? it : b_begin + (it - a_end)) * TK_KEYS;
+        __syncthreads();
+        if (tid < 4) {
+            const int lp = (kt0 + tid * 16) / ps;
+            page_of[tid] = lp < a.table_stride ? table[lp] : -1;
+        }
+        __syncthreads();
+        // raw scores: an item is (key/value head, key); its heads share the key's row
+        for (int item = tid; item < KV * TK_KEYS; item += 256) {
+            const int kvh = item >> 6, jj = item & 63, key = kt0 + jj, page = page_of[jj >> 4];
+            float sc[TK_MAX_REP];
+#pragma unroll
+            for (int r = 0; r < TK_MAX_REP; ++r) sc[r] = 0.f;
+            if (page >= 0 && key <= pos) {
+                const elem_t* kr = a.kpool + (((size_t)page * KV + kvh) * ps + key % ps) * d;
+                for (int c8 = 0; c8 < d; c8 += 8) {
+                    float k8[8];
+                    load8(kr + c8, k8);
+#pragma unroll
+                    for (int r = 0; r < TK_MAX_REP; ++r) {
+                        if (r < rep) {
+                            const float* qr = qs + (kvh * rep + r) * d + c8;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) sc[r] += qr[e] * k8[e];
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < TK_MAX_REP; ++r)
+                if (r < rep) raw[(kvh * rep + r) * TK_KEYS + jj] = sc[r];
+        }
+        __syncthreads();
+        for (int item = tid; item < H * TK_KEYS; item += 256) {
+            const int h = item >> 6, jj = item & 63, key = kt0 + jj;
+            float sc;
+            if (a.talk) {
+                sc = 0.f;
+                for (int g = 0; g < H; ++g) sc += a.talk[h * H + g] * raw[g * TK_KEYS + jj];
+            } else {
+                sc = raw[item];
+            }
+            const bool ok = page_of[jj >> 4] >= 0 && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
+            mix[item] = ok ? sc : -INFINITY;
+        }
+        __syncthreads();
+        for (int h = wave; h < H; h += 4) {
+            const float sc = mix[h * TK_KEYS + lane];
+            const float m_old = head_m[h];
+            const float m_new = fmaxf(m_old, wave_max(sc));
+            const float p = (sc == -INFINITY || m_new == -INFINITY) ? 0.f : expf(sc - m_new);
+            const float sum = wave_sum(p);
+            mix[h * TK_KEYS + lane] = p;
+            if (lane == 0) {
+                const float al = m_old == -INFINITY ? 0.f : expf(m_old - m_new);
+                head_a[h] = al;
+                head_l[h] = head_l[h] * al + sum;
+                head_m[h] = m_new;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < TK_MAX_OUT; ++i) {
+            const int c = tid + i * 256;
+            if (c < n_out) {
+                const int h = c / dv, e = c - h * dv, kvh = h / rep;
+                float sum = 0.f;
+#pragma unroll
+                for (int sub = 0; sub < 4; ++sub) {
+                    const int page = page_of[sub];
+                    if (page < 0) continue;
+                    const elem_t* vr = a.vpool + (((size_t)page * KV + kvh) * dv + e) * ps + (kt0 + sub * 16) % ps;
+                    const float* w = mix + h * TK_KEYS + sub * 16;
+                    float v8[8];
+                    load8(vr, v8);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) sum += w[k] * v8[k];
+                    load8(vr + 8, v8);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) sum += w[8 + k] * v8[k];
+                }
+                acc[i] = acc[i] * head_a[h] + sum;
+            }
+        }
+    }
+    __syncthreads();
+    if (n_split == 1) {
+#pragma unroll
+        for (int i = 0; i < TK_MAX_OUT; ++i) {
+            const int c = tid + i * 256;
+            if (c < n_out) a.out[(size_t)t * n_out + c] = from_f32<elem_t>(acc[i] / head_l[c / dv]);
+        }
+        return;
+    }
+    float* po = part_o + ((size_t)t * n_split + y) * n_out;
+#pragma unroll
+    for (int i = 0; i < TK_MAX_OUT; ++i) {
+        const int c = tid + i * 256;
+        if (c < n_out) po[c] = acc[i];
+    }
+    float* pml = part_ml + ((size_t)t * n_split + y) * H * 2;
+    for (int h = tid; h < H; h += 256) {
+        pml[2 * h] = head_m[h];
+        pml[2 * h + 1] = head_l[h];
+    }
+}
+
+// out[t, h, :] = sum_y part_o[t, y, h, :] e^(m_y - M) / sum_y l_y e^(m_y - M), M = max_y m_y, the shares in order
+__global__ __launch_bounds__(256) void talking_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                            elem_t* __restrict__ out, int n_split, int H, int dv) {
+    const int t = blockIdx.x, n_out = H * dv;
+    for (int c = threadIdx.x; c < n_out; c += 256) {
+        const int h = c / dv;
+        const float* ml = part_ml + (size_t)t * n_split * H * 2 + 2 * h;
+        float M = -INFINITY;
+        for (int y = 0; y < n_split; ++y) M = fmaxf(M, ml[(size_t)y * H * 2]);
+        float L = 0.f, o = 0.f;
+        for (int y = 0; y < n_split; ++y) {
+            const float m = ml[(size_t)y * H * 2];
+            if (m == -INFINITY) continue;
+            const float f = expf(m - M);
+            L += ml[(size_t)y * H * 2 + 1] * f;
+            o += part_o[((size_t)t * n_split + y) * n_out + c] * f;
+        }
+        out[(size_t)t * n_out + c] = from_f32<elem_t>(o / L);
+    }
+}
+
 }  // namespace ms
 
 using namespace ms;
@@ -490,4 +663,35 @@ extern "C" int ms_talking_attention_tiles(const void* q, const void* kpool, cons
 #undef MS_TILE_ND
 #undef MS_TILE
     return check_launch("attention in tiles");
+}
+
+// Whether the kernel whose blocks share a row's keys takes these sizes (else: one block a row, element by element).
+extern "C" int ms_talking_split_takes(int H, int KV, int d, int dv, int ps) {
+    if (H < 1 || KV < 1 || H % KV || H / KV > TK_MAX_REP || d % 8 || ps % 16 || H * dv > 256 * TK_MAX_OUT) return 0;
+    return ((size_t)H * d + 2 * (size_t)H * TK_KEYS + 3 * (size_t)H + 4) * sizeof(float) <= (size_t)TK_MAX_LDS;
+}
+
+// part_o float [T, n_split, H * dv] and part_ml float [T, n_split, H, 2] are the shares' workspace (unused with one share).
+extern "C" int ms_talking_attention_split(const void* q, const void* kpool, const void* vpool, const float* talk, const int* block_table,
+                                          int table_stride, const int* seq_q_start, const int* seq_pos0, int S, void* out, int T, int H,
+                                          int KV, int d, int dv, int ps, int window, int keep_first, float scale, int n_split,
+                                          float* part_o, float* part_ml, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && S > 0, "attention: empty problem");
+    MS_REQUIRE(ms_talking_split_takes(H, KV, d, dv, ps), "attention in shares: %d heads over %d, keys of %d, values of %d, pages of %d are not taken",
+               H, KV, d, dv, ps);
+    MS_REQUIRE(window >= 0 && keep_first >= 0, "attention: window %d, %d first tokens kept", window, keep_first);
+    MS_REQUIRE(n_split >= 1 && n_split <= 256 && (n_split == 1 || (part_o && part_ml)), "attention in shares: %d shares", n_split);
+    MS_REQUIRE(q && kpool && vpool && block_table && seq_q_start && seq_pos0 && out, "attention: a buffer is missing");
+    MS_REQUIRE(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(kpool) | reinterpret_cast<uintptr_t>(vpool)) & 15) == 0,
+               "attention in shares: operands must be 16-byte aligned");
+    TalkArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, talk, block_table, table_stride, seq_q_start, seq_pos0,
+               S, (elem_t*)out, H, KV, d, dv, ps, window, keep_first, scale};
+    const size_t lds = ((size_t)H * d + 2 * (size_t)H * TK_KEYS + 3 * (size_t)H + 4) * sizeof(float);
+    hipLaunchKernelGGL(talking_attention_split_kernel, dim3(T, n_split), dim3(256), lds, stream, a, n_split, part_o, part_ml);
+    if (int rc = check_launch("attention in shares")) return rc;
+    if (n_split > 1) {
+        hipLaunchKernelGGL(talking_merge_kernel, dim3(T), dim3(256), 0, stream, part_o, part_ml, (elem_t*)out, n_split, H, dv);
+        return check_launch("attention merge");
+    }
+    return 0;
 }

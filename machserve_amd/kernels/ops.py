@@ -737,6 +737,21 @@ class HipOps:
                 _ptr(seq_q_len), _ptr(seq_pos0), _c_int(S), _ptr(out), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv),
                 _c_int(page_size), _c_int(window or 0), _c_int(keep_first), _c_float(scale), self._stream()))
             return out
+        if self._plan("ms_talking_split_takes", H, KV, d, dv, page_size, lib=lib):
+            # blocks that share a row's keys, as many as fill the chip: how many follows from the step's rows and the
+            # most 64-position tiles a row can see (its window and first tokens, or the width of the block tables)
+            span = block_table.shape[1] * page_size
+            tiles = -(-span // 64) if not window else min(-(-span // 64), -(-window // 64) + 1 + -(-keep_first // 64))
+            n_split = max(1, min(tiles, -(-2 * self._cus // T), 64))
+            part_o = part_ml = None
+            if n_split > 1:
+                part_o = torch.empty((T, n_split, H * dv), dtype=torch.float32, device=q.device)
+                part_ml = torch.empty((T, n_split, H, 2), dtype=torch.float32, device=q.device)
+            self._check(lib, lib.ms_talking_attention_split(
+                _ptr(q), _ptr(kpool), _ptr(vpool), _ptr(talk), _ptr(block_table), _c_int(block_table.shape[1]), _ptr(seq_q_start),
+                _ptr(seq_pos0), _c_int(S), _ptr(out), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv), _c_int(page_size),
+                _c_int(window or 0), _c_int(keep_first), _c_float(scale), _c_int(n_split), _ptr(part_o), _ptr(part_ml), self._stream()))
+            return out
         self._check(lib, lib.ms_talking_attention(
             _ptr(q), _ptr(kpool), _ptr(vpool), _ptr(talk), _ptr(block_table), _c_int(block_table.shape[1]), _ptr(seq_q_start),
             _ptr(seq_pos0), _c_int(S), _ptr(out), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv), _c_int(page_size),
