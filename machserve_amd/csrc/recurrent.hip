@@ -93,45 +93,85 @@ __global__ __launch_bounds__(256) void dt_softplus_kernel(const float* __restric
 }
 
 // ---- selective scan --------------------------------------------------------------------
-// One thread per (request, channel) with the channel's N states in registers.  Per token:
-// S[n] = exp(dt * A[n]) * S[n] + dt * x * B[t, n];  y = sum_n S[n] * C[t, n] + D * x;  out = y * silu(z).
-template <int NMAX>
-__global__ __launch_bounds__(64) void selective_scan_kernel(const elem_t* __restrict__ x, const elem_t* __restrict__ z, int ldz,
-                                                            const float* __restrict__ dt, const float* __restrict__ dbc, int ldb,
-                                                            int col_b, int col_c, const float* __restrict__ a_log,
-                                                            const float* __restrict__ dskip, float* __restrict__ state,
-                                                            const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
-                                                            const int* __restrict__ seq_slot, elem_t* __restrict__ y, int C, int N) {
-    const int s = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
-    if (c >= C) return;
+// A channel's N states are spread over NL neighbouring lanes (NL a power of two, SPL states a lane), so a wave holds
+// 64 / NL channels and a request's channels fill the chip even where one sequence is all there is.  Per token:
+// S[n] = exp(dt * A[n]) * S[n] + dt * x * B[t, n];  y = sum_n S[n] * C[t, n] + D * x;  out = y * silu(z);
+// the sum over the states is a reduction over the channel's lanes.
+constexpr int SCAN_TILE = 16;
+template <int SPL>
+__global__ __launch_bounds__(256) void selective_scan_kernel(const elem_t* __restrict__ x, const elem_t* __restrict__ z, int ldz,
+                                                             const float* __restrict__ dt, const float* __restrict__ dbc, int ldb,
+                                                             int col_b, int col_c, const float* __restrict__ a_log,
+                                                             const float* __restrict__ dskip, float* __restrict__ state,
+                                                             const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
+                                                             const int* __restrict__ seq_slot, elem_t* __restrict__ y, int C, int N, int NL) {
+    const int s = blockIdx.x, per_block = 256 / NL;
+    const int sub = threadIdx.x % NL, c = blockIdx.y * per_block + threadIdx.x / NL;
+    const bool live = c < C;
+    const int cc = live ? c : C - 1;
     const int q0 = seq_q_start[s], n_rows = seq_q_len[s];
-    float* st = state + ((size_t)seq_slot[s] * C + c) * N;
-    float S[NMAX], A[NMAX];
+    float* st = state + ((size_t)seq_slot[s] * C + cc) * N;
+    float S[SPL], A[SPL];
+    int ns[SPL];
 #pragma unroll
-    for (int n = 0; n < NMAX; ++n) {
-        S[n] = n < N ? st[n] : 0.f;
-        A[n] = n < N ? -expf(a_log[(size_t)c * N + n]) : 0.f;
+    for (int k = 0; k < SPL; ++k) {
+        const int n = sub + k * NL;
+        ns[k] = n < N ? n : -1;
+        S[k] = n < N ? st[n] : 0.f;
+        A[k] = n < N ? -expf(a_log[(size_t)cc * N + n]) : 0.f;
     }
-    const float dsk = dskip ? dskip[c] : 0.f;
-    for (int i = 0; i < n_rows; ++i) {
-        const size_t t = (size_t)(q0 + i);
-        const float d = dt[t * C + c], xv = to_f32(x[t * C + c]), zv = to_f32(z[t * ldz + c]);
-        const float* Bt = dbc + t * ldb + col_b;
-        const float* Ct = dbc + t * ldb + col_c;
-        const float dx = d * xv;
-        float acc = 0.f;
+    const float dsk = dskip ? dskip[cc] : 0.f;
+    // SCAN_TILE tokens' numbers are asked for at once, a tile ahead of the one in use: the walk is one dependent chain,
+    // and a trip to memory per token would be all of its time
+    struct Tile {
+        float d[SCAN_TILE], xv[SCAN_TILE], zv[SCAN_TILE], Bn[SCAN_TILE][SPL], Cn[SCAN_TILE][SPL];
+    };
+    auto fetch = [&](int i0, Tile& tl) {
 #pragma unroll
-        for (int n = 0; n < NMAX; ++n) {
-            if (n < N) {
-                S[n] = expf(d * A[n]) * S[n] + dx * Bt[n];
-                acc += S[n] * Ct[n];
+        for (int j = 0; j < SCAN_TILE; ++j) {
+            const size_t t = (size_t)(q0 + min(i0 + j, n_rows - 1));
+            tl.d[j] = dt[t * C + cc];
+            tl.xv[j] = to_f32(x[t * C + cc]);
+            tl.zv[j] = to_f32(z[t * ldz + cc]);
+#pragma unroll
+            for (int k = 0; k < SPL; ++k) {
+                const int n = ns[k] >= 0 ? ns[k] : 0;
+                tl.Bn[j][k] = dbc[t * ldb + col_b + n];
+                tl.Cn[j][k] = dbc[t * ldb + col_c + n];
             }
         }
-        y[t * C + c] = from_f32<elem_t>((acc + dsk * xv) * silu_f(zv));
-    }
+    };
+    Tile cur, nxt;
+    if (n_rows > 0) fetch(0, cur);
+    for (int i0 = 0; i0 < n_rows; i0 += SCAN_TILE) {
+        if (i0 + SCAN_TILE < n_rows) fetch(i0 + SCAN_TILE, nxt);
 #pragma unroll
-    for (int n = 0; n < NMAX; ++n)
-        if (n < N) st[n] = S[n];
+        for (int j = 0; j < SCAN_TILE; ++j) {
+            if (i0 + j < n_rows) {  // the same for every thread of the block
+                const float d = cur.d[j], xv = cur.xv[j], dx = d * xv;
+                float acc = 0.f;
+#pragma unroll
+                for (int k = 0; k < SPL; ++k) {
+                    if (ns[k] >= 0) {
+#ifdef MS_ELEM_HALF
+                        S[k] = __expf(d * A[k]) * S[k] + dx * cur.Bn[j][k];
+#else
+                        S[k] = expf(d * A[k]) * S[k] + dx * cur.Bn[j][k];
+#endif
+                        acc += S[k] * cur.Cn[j][k];
+                    }
+                }
+                for (int o = NL >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, WAVE);
+                if (sub == 0 && live) y[(size_t)(q0 + i0 + j) * C + c] = from_f32<elem_t>((acc + dsk * xv) * silu_f(cur.zv[j]));
+            }
+        }
+        cur = nxt;
+    }
+    if (live) {
+#pragma unroll
+        for (int k = 0; k < SPL; ++k)
+            if (ns[k] >= 0) st[ns[k]] = S[k];
+    }
 }
 
 // ---- linear attention with a decay per head ---------------------------------------------
@@ -224,26 +264,44 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(const elem_t* __re
             }
         }
     const size_t orow = (size_t)H * dv;
+    // a chunk's rows are asked for a chunk ahead (before their activation), so that the trip to memory runs beside the
+    // chunk in work; thread tid holds elements tid, tid + 256, ... of the [LC][DP] and [LC][VP] tiles
+    constexpr int QN = LC * DP / 256, VN = LC * VP / 256;
+    float qn[QN], kn[QN], vn[VN];
+    auto fetch = [&](int i0) {
+        const int n = min(LC, n_rows - i0);
+#pragma unroll
+        for (int u = 0; u < QN; ++u) {
+            const int idx = tid + u * 256, r = idx / DP, c = idx - r * DP;
+            qn[u] = kn[u] = 0.f;
+            if (r < n && c < d) {
+                const elem_t* row = qkv + (size_t)(q0 + i0 + r) * ld + h * d + c;
+                qn[u] = to_f32(row[col_q]);
+                kn[u] = to_f32(row[col_k]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < VN; ++u) {
+            const int idx = tid + u * 256, r = idx / VP, e = idx - r * VP;
+            vn[u] = (r < n && e < dv) ? to_f32(qkv[(size_t)(q0 + i0 + r) * ld + col_v + h * dv + e]) : 0.f;
+        }
+    };
+    if (n_rows > 0) fetch(0);
     for (int i0 = 0; i0 < n_rows; i0 += LC) {
         const int n = min(LC, n_rows - i0);
         __syncthreads();  // the chunk before has been read
-        for (int idx = tid; idx < LC * DP; idx += 256) {
-            const int r = idx / DP, c = idx - r * DP;
-            float qv = 0.f, kv = 0.f;
-            if (r < n && c < d) {
-                const elem_t* row = qkv + (size_t)(q0 + i0 + r) * ld + h * d + c;
-                qv = silu_f(to_f32(row[col_q]));
-                kv = silu_f(to_f32(row[col_k]));
-            }
-            Qs[idx] = from_f32<elem_t>(qv);
-            Ks[idx] = from_f32<elem_t>(kv);
+#pragma unroll
+        for (int u = 0; u < QN; ++u) {
+            const int idx = tid + u * 256;
+            Qs[idx] = from_f32<elem_t>(silu_f(qn[u]));   // silu(0) = 0: what lies beyond the rows and the head stays zero
+            Ks[idx] = from_f32<elem_t>(silu_f(kn[u]));
         }
-        for (int idx = tid; idx < LC * VP; idx += 256) {
-            const int r = idx / VP, e = idx - r * VP;
-            float v = 0.f;
-            if (r < n && e < dv) v = silu_f(to_f32(qkv[(size_t)(q0 + i0 + r) * ld + col_v + h * dv + e]));
-            VT[e * LC + r] = from_f32<elem_t>(v);
+#pragma unroll
+        for (int u = 0; u < VN; ++u) {
+            const int idx = tid + u * 256, r = idx / VP, e = idx - r * VP;
+            VT[e * LC + r] = from_f32<elem_t>(silu_f(vn[u]));
         }
+        if (i0 + LC < n_rows) fetch(i0 + LC);
         __syncthreads();
         {   // a quarter of the scores a wave: rows rt, columns ct
             const int rt = wave >> 1, ct = wave & 1;
@@ -413,14 +471,14 @@ extern "C" int ms_selective_scan(const void* x, const void* z, int ldz, const fl
     MS_REQUIRE(N <= 128, "selective scan: %d states a channel, at most 128 are built", N);
     MS_REQUIRE(col_b >= 0 && col_c >= 0 && col_b + N <= ldb && col_c + N <= ldb, "selective scan: columns %d, %d of rows of %d", col_b, col_c, ldb);
     MS_REQUIRE(x && z && dt && dbc && a_log && state && seq_q_start && seq_q_len && seq_slot && y, "selective scan: a buffer is missing");
-    const dim3 grid(S, ceil_div(C, 64));
-#define MS_SCAN(NM)                                                                                                          \
-    hipLaunchKernelGGL(selective_scan_kernel<NM>, grid, dim3(64), 0, stream, (const elem_t*)x, (const elem_t*)z, ldz, dt, dbc, \
-                       ldb, col_b, col_c, a_log, dskip, state, seq_q_start, seq_q_len, seq_slot, (elem_t*)y, C, N)
-    if (N <= 16) MS_SCAN(16);
-    else if (N <= 32) MS_SCAN(32);
-    else if (N <= 64) MS_SCAN(64);
-    else MS_SCAN(128);
+    int nl = 1;
+    while (nl < N && nl < 64) nl *= 2;
+    const dim3 grid(S, ceil_div(C, 256 / nl));
+#define MS_SCAN(SP)                                                                                                           \
+    hipLaunchKernelGGL(selective_scan_kernel<SP>, grid, dim3(256), 0, stream, (const elem_t*)x, (const elem_t*)z, ldz, dt, dbc, \
+                       ldb, col_b, col_c, a_log, dskip, state, seq_q_start, seq_q_len, seq_slot, (elem_t*)y, C, N, nl)
+    if (N <= 64) MS_SCAN(1);
+    else MS_SCAN(2);
 #undef MS_SCAN
     return check_launch("selective scan");
 }

@@ -231,29 +231,47 @@ __global__ __launch_bounds__(256) void talking_attention_kernel(TalkArgs a) {
 // taken request by request: the rows of the others are masked, which leaves their sums as they are.
 constexpr float TK_NEG_BIG = -1.0e30f;
 
+// 4 or 8 elements of one row that lie side by side, into elements at .. of a fragment
+__device__ __forceinline__ void frag_set4(Frag& f, int at, const elem_t* p) {
+#ifdef MS_ELEM_HALF
+    const half4_t v = *reinterpret_cast<const half4_t*>(p);
+#else
+    const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+#endif
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f.v[at + i] = v[i];
+}
+
 template <int HPW, int ND, int NT>
 __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a, const int* __restrict__ seq_q_len, int T) {
+    constexpr int NKS = 4, BK = NT * 16;  // heads of up to 128 numbers
     extern __shared__ float lds[];
     const int H = a.H, d = a.d, dv = a.dv, KV = a.KV, rep = H / KV, ps = a.ps;
-    float* raw = lds;                              // [H][16 queries][NT * 16 keys]
+    float* raw = lds;                                // [H][16 queries][NT * 16 keys]
     float* talk_s = raw + (size_t)H * 16 * NT * 16;  // [H][H]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r16 = lane & 15, grp = lane >> 4;
     const int r0 = blockIdx.x * 16, r_end = min(r0 + 16, T);
     const int my_row = min(r0 + r16, T - 1);
     const int h0 = wave * HPW;
-    const int nks = (d + 31) / 32;
+    const bool active = h0 < H;  // a wave beyond the heads only keeps the barriers
     if (a.talk)
         for (int i = tid; i < H * H; i += blockDim.x) talk_s[i] = a.talk[i];
     float m_run[HPW], l_run[HPW];
     f32x4 acc[HPW][ND];
+    Frag qf[HPW][NKS];  // the rows' queries: asked for once
 #pragma unroll
     for (int hh = 0; hh < HPW; ++hh) {
         m_run[hh] = TK_NEG_BIG;
         l_run[hh] = 0.f;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) acc[hh][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const int d0 = ks * 32 + grp * 8;
+            qf[hh][ks] = (h0 + hh < H && d0 < d) ? frag_load(a.q + ((size_t)my_row * H + h0 + hh) * d + d0) : frag_zero();
+        }
     }
-    const elem_t* qrow = a.q + (size_t)my_row * H * d;
+    const int kv0 = min(h0, H - 1) / rep;  // the key/value head of the wave's first head
     int s = seq_of_row(r0, a.seq_q_start, a.S);
     for (; s < a.S && a.seq_q_start[s] < r_end; ++s) {
         const int q0 = a.seq_q_start[s], qn = seq_q_len[s], p0 = a.seq_pos0[s];
@@ -265,127 +283,157 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
         const int lo = a.window > 0 ? max(0, p_lo - a.window + 1) : 0;
         const int n_first = min(a.keep_first, lo);
         const int* table = a.block_table + (size_t)s * a.table_stride;
-        constexpr int BK = NT * 16;
-        const int a_end = (n_first + BK - 1) / BK;     // tiles of the first tokens: [0, a_end)
+        const int a_end = (n_first + BK - 1) / BK;  // tiles of the first tokens: [0, a_end)
         const int b_begin = max(a_end, lo / BK), b_end = p_hi / BK + 1;
         const int n_tiles = a_end + (b_end - b_begin);
-        for (int it = 0; it < n_tiles; ++it) {
-            const int kt0 = (it < a_end ? it : b_begin + (it - a_end)) * BK;
-            int page[NT];
+        auto tile_pos = [&](int it) { return (it < a_end ? it : b_begin + (it - a_end)) * BK; };
+        auto pages_of = [&](int kt0, int* page) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const int lp = (kt0 + nt * 16) / ps;
                 page[nt] = lp < a.table_stride ? table[lp] : -1;
             }
-            // ---- raw scores of this wave's heads
+        };
+        auto load_k = [&](int kvh, const int* page, int kt0, Frag (&kf)[NT][NKS]) {
 #pragma unroll
-            for (int hh = 0; hh < HPW; ++hh) {
-                const int h = h0 + hh;
-                if (h >= H) break;
-                const int kvh = h / rep;
-                f32x4 sc[NT];
+            for (int nt = 0; nt < NT; ++nt) {
+                const int pg = max(page[nt], 0), off = (kt0 + nt * 16) % ps;
+                const elem_t* krow = a.kpool + (((size_t)pg * KV + kvh) * ps + off + r16) * d;
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    sc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-                    const int pg = max(page[nt], 0), off = (kt0 + nt * 16) % ps;
-                    const elem_t* krow = a.kpool + (((size_t)pg * KV + kvh) * ps + off + r16) * d;
-                    for (int ks = 0; ks < nks; ++ks) {
-                        const int d0 = ks * 32 + grp * 8;
-                        const Frag kf = d0 < d ? frag_load(krow + d0) : frag_zero();
-                        const Frag qf = d0 < d ? frag_load(qrow + (size_t)h * d + d0) : frag_zero();
-                        mma_16x16x32(sc[nt], kf, qf);
-                    }
-                    if (a.talk) {
-                        float* dst = raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4;
-                        *reinterpret_cast<f32x4*>(dst) = sc[nt] * a.scale;
-                    }
+                for (int ks = 0; ks < NKS; ++ks) {
+                    const int d0 = ks * 32 + grp * 8;
+                    kf[nt][ks] = d0 < d ? frag_load(krow + d0) : frag_zero();
                 }
-                if (!a.talk) {  // no exchange: the head's own scores stay in registers (see below)
+            }
+        };
+        auto load_v = [&](int kvh, const int* page, int kt0, Frag (&vf)[ND]) {
+#pragma unroll
+            for (int dt = 0; dt < ND; ++dt) {
+                const int e = dt * 16 + r16;
+                vf[dt] = frag_zero();
+                if (e < dv) {
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt) {
-                        float* dst = raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4;
-                        *reinterpret_cast<f32x4*>(dst) = sc[nt] * a.scale;
+                        const int pg = max(page[nt], 0), off = (kt0 + nt * 16) % ps + grp * 4;
+                        frag_set4(vf[dt], nt * 4, a.vpool + (((size_t)pg * KV + kvh) * dv + e) * ps + off);
+                    }
+                }
+            }
+        };
+        int page[NT], page_n[NT];
+        Frag kf[NT][NKS], kf_n[NT][NKS], vf[ND];
+        if (active) {
+            pages_of(tile_pos(0), page);
+            load_k(kv0, page, tile_pos(0), kf);
+        }
+        for (int it = 0; it < n_tiles; ++it) {
+            const int kt0 = tile_pos(it);
+            if (active) {
+                // this tile's values and the next tile's keys are asked for now and used later
+                load_v(kv0, page, kt0, vf);
+                if (it + 1 < n_tiles) {
+                    pages_of(tile_pos(it + 1), page_n);
+                    load_k(kv0, page_n, tile_pos(it + 1), kf_n);
+                }
+                // ---- raw scores of this wave's heads
+                int kv_have = kv0;
+#pragma unroll
+                for (int hh = 0; hh < HPW; ++hh) {
+                    const int h = h0 + hh;
+                    if (h >= H) break;
+                    if (h / rep != kv_have) {
+                        kv_have = h / rep;
+                        load_k(kv_have, page, kt0, kf);
+                    }
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) {
+                        f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int ks = 0; ks < NKS; ++ks)
+                            if (ks * 32 < d) mma_16x16x32(sc, kf[nt][ks], qf[hh][ks]);
+                        *reinterpret_cast<f32x4*>(raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4) = sc * a.scale;
                     }
                 }
             }
             __syncthreads();
-            // ---- exchange, softmax, values
+            if (active) {
+                // ---- exchange, softmax, values
+                int v_have = kv0;
 #pragma unroll
-            for (int hh = 0; hh < HPW; ++hh) {
-                const int h = h0 + hh;
-                if (h >= H) break;
-                const int kvh = h / rep;
-                f32x4 mixed[NT];
+                for (int hh = 0; hh < HPW; ++hh) {
+                    const int h = h0 + hh;
+                    if (h >= H) break;
+                    if (h / rep != v_have) {
+                        v_have = h / rep;
+                        load_v(v_have, page, kt0, vf);
+                    }
+                    f32x4 mixed[NT];
+                    if (a.talk) {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) mixed[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-                if (a.talk) {
-                    for (int g = 0; g < H; ++g) {
-                        const float w = talk_s[h * H + g];
+                        for (int nt = 0; nt < NT; ++nt) mixed[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                        for (int g = 0; g < H; ++g) {
+                            const float w = talk_s[h * H + g];
+#pragma unroll
+                            for (int nt = 0; nt < NT; ++nt)
+                                mixed[nt] += w * *reinterpret_cast<const f32x4*>(raw + (((size_t)g * 16 + r16) * NT + nt) * 16 + grp * 4);
+                        }
+                    } else {
 #pragma unroll
                         for (int nt = 0; nt < NT; ++nt)
-                            mixed[nt] += w * *reinterpret_cast<const f32x4*>(raw + (((size_t)g * 16 + r16) * NT + nt) * 16 + grp * 4);
+                            mixed[nt] = *reinterpret_cast<const f32x4*>(raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4);
                     }
-                } else {
+                    bool ok[NT][4];
+                    float tmax = TK_NEG_BIG;
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt)
-                        mixed[nt] = *reinterpret_cast<const f32x4*>(raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4);
-                }
-                bool ok[NT][4];
-                float tmax = TK_NEG_BIG;
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int key = kt0 + nt * 16 + grp * 4 + i;
-                        ok[nt][i] = mine && page[nt] >= 0 && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
-                        if (ok[nt][i]) tmax = fmaxf(tmax, mixed[nt][i]);
-                    }
-                tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
-                tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-                const float m_new = fmaxf(m_run[hh], tmax);
-                float psum = 0.f;
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float p = ok[nt][i] ? expf(mixed[nt][i] - m_new) : 0.f;
-                        mixed[nt][i] = p;
-                        psum += p;
-                    }
-                psum += __shfl_xor(psum, 16, WAVE);
-                psum += __shfl_xor(psum, 32, WAVE);
-                const float alpha = expf(m_run[hh] - m_new);
-                l_run[hh] = l_run[hh] * alpha + psum;
-                m_run[hh] = m_new;
-                Frag pf;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    pf.v[i] = from_f32<elem_t>(mixed[0][i]);
-                    pf.v[4 + i] = from_f32<elem_t>(NT > 1 ? mixed[NT - 1][i] : 0.f);
-                }
-#pragma unroll
-                for (int dt = 0; dt < ND; ++dt) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) acc[hh][dt][i] *= alpha;
-                    const int e = dt * 16 + r16;
-                    Frag vf = frag_zero();
-                    if (e < dv) {
-#pragma unroll
-                        for (int nt = 0; nt < NT; ++nt) {
-                            const int pg = max(page[nt], 0), off = (kt0 + nt * 16) % ps + grp * 4;
-                            const elem_t* v0 = a.vpool + (((size_t)pg * KV + kvh) * dv + e) * ps + off;
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) vf.v[nt * 4 + i] = v0[i];
+                        for (int i = 0; i < 4; ++i) {
+                            const int key = kt0 + nt * 16 + grp * 4 + i;
+                            ok[nt][i] = mine && page[nt] >= 0 && key <= pos && (a.window <= 0 || pos - key < a.window || key < a.keep_first);
+                            if (ok[nt][i]) tmax = fmaxf(tmax, mixed[nt][i]);
                         }
+                    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+                    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+                    const float m_new = fmaxf(m_run[hh], tmax);
+                    float psum = 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float p = ok[nt][i] ? expf(mixed[nt][i] - m_new) : 0.f;
+                            mixed[nt][i] = p;
+                            psum += p;
+                        }
+                    psum += __shfl_xor(psum, 16, WAVE);
+                    psum += __shfl_xor(psum, 32, WAVE);
+                    const float alpha = expf(m_run[hh] - m_new);
+                    l_run[hh] = l_run[hh] * alpha + psum;
+                    m_run[hh] = m_new;
+                    Frag pf;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        pf.v[i] = from_f32<elem_t>(mixed[0][i]);
+                        pf.v[4 + i] = from_f32<elem_t>(NT > 1 ? mixed[NT - 1][i] : 0.f);
                     }
-                    mma_16x16x32(acc[hh][dt], vf, pf);
+#pragma unroll
+                    for (int dt = 0; dt < ND; ++dt) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) acc[hh][dt][i] *= alpha;
+                        mma_16x16x32(acc[hh][dt], vf[dt], pf);
+                    }
                 }
             }
             __syncthreads();
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                page[nt] = page_n[nt];
+#pragma unroll
+                for (int ks = 0; ks < NKS; ++ks) kf[nt][ks] = kf_n[nt][ks];
+            }
         }
     }
     // O^T: lane holds value columns dt * 16 + grp * 4 + i of query r16
-    if (r0 + r16 < T) {
+    if (r0 + r16 < T && active) {
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
             const int h = h0 + hh;
@@ -619,9 +667,9 @@ extern "C" int ms_talking_attention(const void* q, const void* kpool, const void
 }
 
 // Whether the tile kernel takes these sizes (else the kernel of one row a block runs): head sizes that are multiples
-// of 8, at most 32 heads of at most 128 values, pages of a multiple of 16 positions.
+// of 8 up to 128, at most 32 heads of at most 128 values (a multiple of 4), pages of a multiple of 16 positions.
 extern "C" int ms_talking_tile_takes(int H, int KV, int d, int dv, int ps) {
-    if (H < 1 || KV < 1 || H % KV || d % 8 || d > 256 || dv > 128 || dv < 1 || ps % 16 || H > 32) return 0;
+    if (H < 1 || KV < 1 || H % KV || d % 8 || d > 128 || dv > 128 || dv < 1 || dv % 4 || ps % 16 || H > 32) return 0;
     const int nt = H <= 20 ? 2 : 1;
     return ((size_t)H * 16 * nt * 16 + (size_t)H * H) * sizeof(float) <= (size_t)TK_MAX_LDS;
 }
