@@ -151,8 +151,18 @@ __global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ x, co
     const size_t r = blockIdx.x;
     float ss = 0.f;
     for (int c = threadIdx.x; c < d; c += 256) {
+        // eight sums are asked for at once and added in order: one trip to memory for eight, not eight trips
+        const float* src = partials + r * d + c;
         float v = 0.f;
-        for (int p = 0; p < n_partials; ++p) v += partials[p * partial_stride + r * d + c];
+        int p = 0;
+        for (; p + 8 <= n_partials; p += 8) {
+            float q[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) q[k] = src[(size_t)(p + k) * partial_stride];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v += q[k];
+        }
+        for (; p < n_partials; ++p) v += src[(size_t)p * partial_stride];
         vals[c] = v;
         ss += v * v;
     }

@@ -82,6 +82,7 @@ __global__ __launch_bounds__(256) void dt_softplus_kernel(const float* __restric
     const float bias = b ? b[c] : 0.f;
 #pragma unroll
     for (int k = 0; k < DT_ROWS; ++k) acc[k] = bias;
+#pragma unroll 8
     for (int r = 0; r < R; ++r) {
         const float w = wt[(size_t)r * C + c];
 #pragma unroll
@@ -98,28 +99,40 @@ __global__ __launch_bounds__(256) void dt_softplus_kernel(const float* __restric
 // S[n] = exp(dt * A[n]) * S[n] + dt * x * B[t, n];  y = sum_n S[n] * C[t, n] + D * x;  out = y * silu(z);
 // the sum over the states is a reduction over the channel's lanes.
 constexpr int SCAN_TILE = 16;
+// A request's rows in one walk; or cut into chunks that are walked side by side: first each from zero (what it adds),
+// then, after the states that come into the chunks are known (scan_carry_kernel), each from its own.
+enum ScanMode { SCAN_WHOLE = 0, SCAN_LOCAL = 1, SCAN_FINAL = 2 };
 template <int SPL>
 __global__ __launch_bounds__(256) void selective_scan_kernel(const elem_t* __restrict__ x, const elem_t* __restrict__ z, int ldz,
                                                              const float* __restrict__ dt, const float* __restrict__ dbc, int ldb,
                                                              int col_b, int col_c, const float* __restrict__ a_log,
                                                              const float* __restrict__ dskip, float* __restrict__ state,
                                                              const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
-                                                             const int* __restrict__ seq_slot, elem_t* __restrict__ y, int C, int N, int NL) {
+                                                             const int* __restrict__ seq_slot, elem_t* __restrict__ y, int C, int N, int NL,
+                                                             int mode, int chunk_len, int n_chunks, float* __restrict__ carry,
+                                                             float* __restrict__ csum) {
     const int s = blockIdx.x, per_block = 256 / NL;
     const int sub = threadIdx.x % NL, c = blockIdx.y * per_block + threadIdx.x / NL;
     const bool live = c < C;
     const int cc = live ? c : C - 1;
-    const int q0 = seq_q_start[s], n_rows = seq_q_len[s];
+    const int q0 = seq_q_start[s] + (mode == SCAN_WHOLE ? 0 : blockIdx.z * chunk_len);
+    const int left = seq_q_len[s] - (mode == SCAN_WHOLE ? 0 : blockIdx.z * chunk_len);
+    if (left <= 0) return;  // the same for every thread of the block
+    const int n_rows = mode == SCAN_WHOLE ? left : min(left, chunk_len);
+    const bool last = n_rows == left;
+    if (mode == SCAN_LOCAL && last) return;  // nobody needs what the last chunk passes on
     float* st = state + ((size_t)seq_slot[s] * C + cc) * N;
+    float* pass = mode == SCAN_WHOLE ? nullptr : carry + (((size_t)s * n_chunks + blockIdx.z) * C + cc) * N;
     float S[SPL], A[SPL];
     int ns[SPL];
 #pragma unroll
     for (int k = 0; k < SPL; ++k) {
         const int n = sub + k * NL;
         ns[k] = n < N ? n : -1;
-        S[k] = n < N ? st[n] : 0.f;
+        S[k] = n >= N || mode == SCAN_LOCAL ? 0.f : mode == SCAN_WHOLE ? st[n] : pass[n];
         A[k] = n < N ? -expf(a_log[(size_t)cc * N + n]) : 0.f;
     }
+    float dsum = 0.f;
     const float dsk = dskip ? dskip[cc] : 0.f;
     // SCAN_TILE tokens' numbers are asked for at once, a tile ahead of the one in use: the walk is one dependent chain,
     // and a trip to memory per token would be all of its time
@@ -149,6 +162,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const elem_t* __res
         for (int j = 0; j < SCAN_TILE; ++j) {
             if (i0 + j < n_rows) {  // the same for every thread of the block
                 const float d = cur.d[j], xv = cur.xv[j], dx = d * xv;
+                dsum += d;
                 float acc = 0.f;
 #pragma unroll
                 for (int k = 0; k < SPL; ++k) {
@@ -161,16 +175,45 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const elem_t* __res
                         acc += S[k] * cur.Cn[j][k];
                     }
                 }
-                for (int o = NL >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, WAVE);
-                if (sub == 0 && live) y[(size_t)(q0 + i0 + j) * C + c] = from_f32<elem_t>((acc + dsk * xv) * silu_f(cur.zv[j]));
+                if (mode != SCAN_LOCAL) {  // the same for every thread
+                    for (int o = NL >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, WAVE);
+                    if (sub == 0 && live) y[(size_t)(q0 + i0 + j) * C + c] = from_f32<elem_t>((acc + dsk * xv) * silu_f(cur.zv[j]));
+                }
             }
         }
         cur = nxt;
     }
-    if (live) {
+    if (!live) return;
+    if (mode == SCAN_LOCAL) {  // what the chunk adds to a state that comes in, and the sum of its step sizes
+#pragma unroll
+        for (int k = 0; k < SPL; ++k)
+            if (ns[k] >= 0) pass[ns[k]] = S[k];
+        if (sub == 0) csum[((size_t)s * n_chunks + blockIdx.z) * C + c] = dsum;
+    } else if (mode == SCAN_WHOLE || last) {
 #pragma unroll
         for (int k = 0; k < SPL; ++k)
             if (ns[k] >= 0) st[ns[k]] = S[k];
+    }
+}
+
+// Between the two passes over the chunks: carry[s, ch] holds what chunk ch adds from zero and receives the state that
+// comes into it, S_in(ch + 1) = exp(A * sum of the chunk's step sizes) * S_in(ch) + what it adds.
+__global__ __launch_bounds__(256) void scan_carry_kernel(const float* __restrict__ a_log, const float* __restrict__ state,
+                                                         const int* __restrict__ seq_q_len, const int* __restrict__ seq_slot,
+                                                         float* __restrict__ carry, const float* __restrict__ csum, int C, int N,
+                                                         int chunk_len, int n_chunks) {
+    const int s = blockIdx.x;
+    const size_t idx = (size_t)blockIdx.y * 256 + threadIdx.x;
+    if (idx >= (size_t)C * N) return;
+    const int c = (int)(idx / N);
+    const int nch = (seq_q_len[s] + chunk_len - 1) / chunk_len;
+    const float A = -expf(a_log[idx]);
+    float Sin = state[(size_t)seq_slot[s] * C * N + idx];
+    for (int ch = 0; ch < nch; ++ch) {
+        float* p = carry + ((size_t)s * n_chunks + ch) * C * N + idx;
+        const float add = ch + 1 < nch ? *p : 0.f;
+        *p = Sin;
+        if (ch + 1 < nch) Sin = expf(A * csum[((size_t)s * n_chunks + ch) * C + c]) * Sin + add;
     }
 }
 
@@ -465,20 +508,35 @@ extern "C" int ms_dt_softplus(const float* dbc, int ldb, const float* w, const f
 
 extern "C" int ms_selective_scan(const void* x, const void* z, int ldz, const float* dt, const float* dbc, int ldb, int col_b,
                                  int col_c, const float* a_log, const float* dskip, float* state, const int* seq_q_start,
-                                 const int* seq_q_len, const int* seq_slot, int S, void* y, int T, int C, int N,
-                                 hipStream_t stream) {
+                                 const int* seq_q_len, const int* seq_slot, int S, void* y, int T, int C, int N, int chunk_len,
+                                 int n_chunks, float* carry, float* csum, hipStream_t stream) {
     MS_REQUIRE(T > 0 && S > 0 && C > 0 && N > 0, "selective scan: T=%d S=%d C=%d N=%d", T, S, C, N);
     MS_REQUIRE(N <= 128, "selective scan: %d states a channel, at most 128 are built", N);
     MS_REQUIRE(col_b >= 0 && col_c >= 0 && col_b + N <= ldb && col_c + N <= ldb, "selective scan: columns %d, %d of rows of %d", col_b, col_c, ldb);
     MS_REQUIRE(x && z && dt && dbc && a_log && state && seq_q_start && seq_q_len && seq_slot && y, "selective scan: a buffer is missing");
+    MS_REQUIRE(chunk_len == 0 || (chunk_len > 0 && n_chunks > 0 && carry && csum), "selective scan: chunks of %d need their workspace", chunk_len);
     int nl = 1;
     while (nl < N && nl < 64) nl *= 2;
-    const dim3 grid(S, ceil_div(C, 256 / nl));
-#define MS_SCAN(SP)                                                                                                           \
-    hipLaunchKernelGGL(selective_scan_kernel<SP>, grid, dim3(256), 0, stream, (const elem_t*)x, (const elem_t*)z, ldz, dt, dbc, \
-                       ldb, col_b, col_c, a_log, dskip, state, seq_q_start, seq_q_len, seq_slot, (elem_t*)y, C, N, nl)
-    if (N <= 64) MS_SCAN(1);
-    else MS_SCAN(2);
+#define MS_SCAN(SP, MODE, Z)                                                                                                       \
+    hipLaunchKernelGGL(selective_scan_kernel<SP>, dim3(S, ceil_div(C, 256 / nl), Z), dim3(256), 0, stream, (const elem_t*)x,          \
+                       (const elem_t*)z, ldz, dt, dbc, ldb, col_b, col_c, a_log, dskip, state, seq_q_start, seq_q_len, seq_slot,     \
+                       (elem_t*)y, C, N, nl, MODE, chunk_len, n_chunks, carry, csum)
+#define MS_SCAN_N(MODE, Z)            \
+    do {                              \
+        if (N <= 64) MS_SCAN(1, MODE, Z); \
+        else MS_SCAN(2, MODE, Z);     \
+    } while (0)
+    if (chunk_len == 0) {
+        MS_SCAN_N(SCAN_WHOLE, 1);
+    } else {
+        MS_SCAN_N(SCAN_LOCAL, n_chunks);
+        if (int rc = check_launch("selective scan, chunks from zero")) return rc;
+        hipLaunchKernelGGL(scan_carry_kernel, dim3(S, (unsigned)ceil_div((long)C * N, 256L)), dim3(256), 0, stream, a_log, state, seq_q_len,
+                           seq_slot, carry, csum, C, N, chunk_len, n_chunks);
+        if (int rc = check_launch("selective scan, states between chunks")) return rc;
+        MS_SCAN_N(SCAN_FINAL, n_chunks);
+    }
+#undef MS_SCAN_N
 #undef MS_SCAN
     return check_launch("selective scan");
 }

@@ -603,24 +603,36 @@ __global__ __launch_bounds__(256) void talking_attention_split_kernel(TalkArgs a
     }
 }
 
-// out[t, h, :] = sum_y part_o[t, y, h, :] e^(m_y - M) / sum_y l_y e^(m_y - M), M = max_y m_y, the shares in order
-__global__ __launch_bounds__(256) void talking_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+// out[t, h, :] = sum_y part_o[t, y, h, :] e^(m_y - M) / sum_y l_y e^(m_y - M), M = max_y m_y, the shares in order.
+// A block is one (row, head): the shares' factors are worked out once, then every thread sums its columns over the
+// shares with nothing between the loads.
+__global__ __launch_bounds__(128) void talking_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                             elem_t* __restrict__ out, int n_split, int H, int dv) {
-    const int t = blockIdx.x, n_out = H * dv;
-    for (int c = threadIdx.x; c < n_out; c += 256) {
-        const int h = c / dv;
-        const float* ml = part_ml + (size_t)t * n_split * H * 2 + 2 * h;
+    __shared__ float fac[256];
+    __shared__ float inv_l;
+    const int t = blockIdx.x, h = blockIdx.y, n_out = H * dv;
+    const float* ml = part_ml + (size_t)t * n_split * H * 2 + 2 * h;
+    if (threadIdx.x < 64) {
         float M = -INFINITY;
-        for (int y = 0; y < n_split; ++y) M = fmaxf(M, ml[(size_t)y * H * 2]);
-        float L = 0.f, o = 0.f;
-        for (int y = 0; y < n_split; ++y) {
+        for (int y = threadIdx.x; y < n_split; y += 64) M = fmaxf(M, ml[(size_t)y * H * 2]);
+        M = wave_max(M);
+        float L = 0.f;
+        for (int y = threadIdx.x; y < n_split; y += 64) {
             const float m = ml[(size_t)y * H * 2];
-            if (m == -INFINITY) continue;
-            const float f = expf(m - M);
+            const float f = m == -INFINITY ? 0.f : expf(m - M);
+            fac[y] = f;
             L += ml[(size_t)y * H * 2 + 1] * f;
-            o += part_o[((size_t)t * n_split + y) * n_out + c] * f;
         }
-        out[(size_t)t * n_out + c] = from_f32<elem_t>(o / L);
+        L = wave_sum(L);
+        if (threadIdx.x == 0) inv_l = 1.0f / L;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < dv; e += 128) {
+        const float* po = part_o + (size_t)t * n_split * n_out + (size_t)h * dv + e;
+        float o = 0.f;
+#pragma unroll 8
+        for (int y = 0; y < n_split; ++y) o += po[(size_t)y * n_out] * fac[y];
+        out[(size_t)t * n_out + (size_t)h * dv + e] = from_f32<elem_t>(o * inv_l);
     }
 }
 
@@ -738,7 +750,7 @@ extern "C" int ms_talking_attention_split(const void* q, const void* kpool, cons
     hipLaunchKernelGGL(talking_attention_split_kernel, dim3(T, n_split), dim3(256), lds, stream, a, n_split, part_o, part_ml);
     if (int rc = check_launch("attention in shares")) return rc;
     if (n_split > 1) {
-        hipLaunchKernelGGL(talking_merge_kernel, dim3(T), dim3(256), 0, stream, part_o, part_ml, (elem_t*)out, n_split, H, dv);
+        hipLaunchKernelGGL(talking_merge_kernel, dim3(T, H), dim3(128), 0, stream, part_o, part_ml, (elem_t*)out, n_split, H, dv);
         return check_launch("attention merge");
     }
     return 0;

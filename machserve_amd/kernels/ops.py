@@ -593,6 +593,9 @@ class HipOps:
                                             _c_int(taps), self._stream()))
         return out
 
+    SCAN_CHUNK = 64           # tokens of a chunk of the scan
+    SCAN_CHUNK_MIN_ROWS = 256  # steps of at least this many rows, half as many a request on average, are cut into chunks
+
     def selective_scan(self, x: torch.Tensor, xz: torch.Tensor, dbc: torch.Tensor, dt_rank: int, n_states: int, w_dt: torch.Tensor,
                        b_dt: Optional[torch.Tensor], a_log: torch.Tensor, d_skip: Optional[torch.Tensor], state: torch.Tensor,
                        seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor) -> torch.Tensor:
@@ -619,10 +622,22 @@ class HipOps:
                                             _c_int(dt_rank), self._stream()))
         y = torch.empty((T, C), dtype=self.dtype, device=x.device)
         z = _c_void(xz.data_ptr() + C * xz.element_size())
+        # Long portions are cut into chunks that are walked side by side (each from zero, then each from the state that
+        # comes into it): one walk over a long prompt keeps a sixteenth of the chip busy.  The cut follows from the
+        # step's rows and requests alone.
+        chunk = n_chunks = 0
+        carry = csum = None
+        if T >= self.SCAN_CHUNK_MIN_ROWS and T // S >= self.SCAN_CHUNK_MIN_ROWS // 2:
+            n_chunks = -(-T // self.SCAN_CHUNK)
+            if S * n_chunks * C * n_states * 4 <= (256 << 20):
+                chunk = self.SCAN_CHUNK
+                carry = torch.empty((S, n_chunks, C, n_states), dtype=torch.float32, device=x.device)
+                csum = torch.empty((S, n_chunks, C), dtype=torch.float32, device=x.device)
         self._check(lib, lib.ms_selective_scan(_ptr(x), z, _c_int(2 * C), _ptr(dt), _ptr(dbc), _c_int(ldb), _c_int(dt_rank),
                                                _c_int(dt_rank + n_states), _ptr(a_log), _ptr(d_skip), _ptr(state), _ptr(seq_q_start),
                                                _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(y), _c_int(T), _c_int(C),
-                                               _c_int(n_states), self._stream()))
+                                               _c_int(n_states), _c_int(chunk), _c_int(n_chunks if chunk else 0), _ptr(carry), _ptr(csum),
+                                               self._stream()))
         return y
 
     def lightning_attention(self, qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.Tensor, state: torch.Tensor,

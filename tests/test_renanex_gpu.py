@@ -117,6 +117,31 @@ def test_selective_scan_in_one_step_and_in_many(dtype, C, N, R):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_a_long_scan_in_chunks_equals_the_walk_token_after_token(dtype):
+    """Steps of many rows cut their requests into chunks that are walked side by side; the result is the one walk's."""
+    ops = ops_of(dtype)
+    torch.manual_seed(5)
+    C, N, R, lens = 48, 12, 3, [300, 1, 129, 210]
+    T = sum(lens)
+    assert T >= ops.SCAN_CHUNK_MIN_ROWS and T // len(lens) >= ops.SCAN_CHUNK_MIN_ROWS // 2
+    x, z = (torch.randn(T, C).to(dtype).float() for _ in range(2))
+    dbc = torch.randn(T, R + 2 * N)
+    w_dt, b_dt, a_log, dsk = torch.randn(C, R) * 0.5, torch.randn(C) - 2.0, torch.randn(C, N) * 0.5, torch.randn(C)
+    start = torch.randn(6, C, N)
+    slots, starts = [4, 0, 2, 5], [0, 300, 301, 430]
+    args = lambda rows: (dev(x[rows], dtype), dev(torch.cat([torch.zeros(T, C), z], 1)[rows], dtype), dev(dbc[rows]), R, N, dev(w_dt.t()),
+                         dev(b_dt), dev(a_log), dev(dsk))
+    state = dev(start.clone())
+    got = ops.selective_scan(*args(slice(0, T)), state, i32(starts), i32(lens), i32(slots))
+    for s, (q0, n) in enumerate(zip(starts, lens)):     # each request alone, token after token
+        alone = dev(start.clone())
+        want = torch.cat([ops.selective_scan(*args(slice(t, t + 1)), alone, i32([0]), i32([1]), i32([slots[s]])) for t in range(q0, q0 + n)])
+        close(got[q0:q0 + n], want, dtype, f"request {s} in chunks")
+        close(state[slots[s]], alone[slots[s]], torch.float32, f"state of request {s}")
+    assert torch.equal(state[1].cpu(), start[1]) and torch.equal(state[3].cpu(), start[3])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("chunked", [False, True])
 @pytest.mark.parametrize("H,d,dv", [(2, 16, 24), (1, 40, 8), (3, 8, 70), (2, 72, 16), (2, 128, 128), (1, 136, 8)])
 def test_lightning_attention_in_one_step_and_in_many(dtype, H, d, dv, chunked):
