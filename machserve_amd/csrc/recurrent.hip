@@ -281,7 +281,8 @@ template <int DT, int CT>
 __global__ __launch_bounds__(256) void lightning_chunk_kernel(const elem_t* __restrict__ qkv, int ld, int col_q, int col_k, int col_v,
                                                               const float* __restrict__ decay, float* __restrict__ state,
                                                               const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
-                                                              const int* __restrict__ seq_slot, float* __restrict__ o, int H, int d, int dv) {
+                                                              const int* __restrict__ seq_slot, float* __restrict__ o, int H, int d, int dv,
+                                                              int mode, int seg_len, int n_segs, float* __restrict__ carry) {
     constexpr int DP = DT * 16, VP = CT * 64;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     elem_t* Qs = reinterpret_cast<elem_t*>(smem);  // [LC][DP]
@@ -290,8 +291,16 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(const elem_t* __re
     elem_t* Ps = VT + VP * LC;                     // [LC][LC]: scores times decays
     float* pw = reinterpret_cast<float*>(Ps + LC * LC);  // [LC + 1]: decay^k
     const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r16 = lane & 15, grp = lane >> 4;
-    const int q0 = seq_q_start[s], n_rows = seq_q_len[s];
-    float* st = state + (((size_t)seq_slot[s] * H + h) * d) * dv;
+    // a request's rows in one walk (SCAN_WHOLE), or in segments of seg_len rows (a multiple of the chunk) that are walked
+    // side by side: first each from zero, leaving what it adds (SCAN_LOCAL), then each from the state that comes into it
+    const int seg0 = mode == SCAN_WHOLE ? 0 : blockIdx.z * seg_len;
+    const int left = seq_q_len[s] - seg0;
+    if (left <= 0) return;
+    const int q0 = seq_q_start[s] + seg0, n_rows = mode == SCAN_WHOLE ? left : min(left, seg_len);
+    const bool last = n_rows == left;
+    if (mode == SCAN_LOCAL && last) return;
+    float* st = mode == SCAN_WHOLE ? state + (((size_t)seq_slot[s] * H + h) * d) * dv
+                                   : carry + ((((size_t)s * n_segs + blockIdx.z) * H + h) * d) * dv;
     const float lam = decay[h];
     if (tid <= LC) pw[tid] = powf(lam, (float)tid);
     f32x4 S[DT][CT];
@@ -303,7 +312,7 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(const elem_t* __re
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int dd = dt * 16 + grp * 4 + i;
-                S[dt][c][i] = (dd < d && e < dv) ? st[(size_t)dd * dv + e] : 0.f;
+                S[dt][c][i] = (dd < d && e < dv && mode != SCAN_LOCAL) ? st[(size_t)dd * dv + e] : 0.f;
             }
         }
     const size_t orow = (size_t)H * dv;
@@ -418,7 +427,7 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(const elem_t* __re
 #pragma unroll
                 for (int ii = 0; ii < 4; ++ii) {
                     const int i = rt * 16 + grp * 4 + ii;
-                    if (i < n && e < dv) o[(size_t)(q0 + i0 + i) * orow + (size_t)h * dv + e] = O[rt][c][ii];
+                    if (i < n && e < dv && mode != SCAN_LOCAL) o[(size_t)(q0 + i0 + i) * orow + (size_t)h * dv + e] = O[rt][c][ii];
                 }
             }
         // the state after the chunk
@@ -441,6 +450,9 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(const elem_t* __re
             }
         }
     }
+    // the state after the rows: into the workspace what a segment adds; into the request's slot after its last row
+    float* dst = mode == SCAN_LOCAL ? st : (mode == SCAN_WHOLE || last) ? state + (((size_t)seq_slot[s] * H + h) * d) * dv : nullptr;
+    if (dst == nullptr) return;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -449,9 +461,27 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(const elem_t* __re
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int dd = dt * 16 + grp * 4 + i;
-                if (dd < d && e < dv) st[(size_t)dd * dv + e] = S[dt][c][i];
+                if (dd < d && e < dv) dst[(size_t)dd * dv + e] = S[dt][c][i];
             }
         }
+}
+
+// Between the two passes over the segments: carry[s, g, h] holds what segment g adds from zero and receives the state
+// that comes into it, S_in(g + 1) = decay^(rows of g) * S_in(g) + what g adds.
+__global__ __launch_bounds__(256) void lightning_carry_kernel(const float* __restrict__ decay, const float* __restrict__ state,
+                                                              const int* __restrict__ seq_q_len, const int* __restrict__ seq_slot,
+                                                              float* __restrict__ carry, int H, int per_head, int seg_len, int n_segs) {
+    const int s = blockIdx.x, h = blockIdx.y, i = blockIdx.z * 256 + threadIdx.x;
+    if (i >= per_head) return;
+    const int n = seq_q_len[s], segs = (n + seg_len - 1) / seg_len;
+    const float f = powf(decay[h], (float)seg_len);  // every segment that passes something on is a whole one
+    float Sin = state[((size_t)seq_slot[s] * H + h) * per_head + i];
+    for (int g = 0; g < segs; ++g) {
+        float* p = carry + (((size_t)s * n_segs + g) * H + h) * per_head + i;
+        const float add = g + 1 < segs ? *p : 0.f;
+        *p = Sin;
+        if (g + 1 < segs) Sin = f * Sin + add;
+    }
 }
 
 // out[t, :] = o[t, :] / sqrt(mean(o[t, :]^2) + eps) * w * sigmoid(gate[t, :])
@@ -572,26 +602,43 @@ extern "C" int ms_gated_rmsnorm(const float* o, const void* gate, int ldg, const
 // Whether the kernel that walks a request in chunks on the matrix cores takes these head sizes.
 extern "C" int ms_lightning_chunked_takes(int d, int dv) { return d >= 1 && d <= 128 && dv >= 1 && dv <= 128; }
 
+// seg_len > 0 (a multiple of 32): the requests' rows in segments walked side by side, with carry float
+// [S, n_segs, H, d, dv] as workspace; 0: each request in one walk.
 extern "C" int ms_lightning_chunked(const void* qkv, int ld, int col_q, int col_k, int col_v, const float* decay, float* state,
                                     const int* seq_q_start, const int* seq_q_len, const int* seq_slot, int S, float* o, int T, int H,
-                                    int d, int dv, hipStream_t stream) {
+                                    int d, int dv, int seg_len, int n_segs, float* carry, hipStream_t stream) {
     MS_REQUIRE(T > 0 && S > 0 && H > 0, "lightning attention: T=%d S=%d H=%d", T, S, H);
     MS_REQUIRE(ms_lightning_chunked_takes(d, dv), "lightning attention in chunks: heads of %d and values of %d are not taken", d, dv);
     MS_REQUIRE(col_q >= 0 && col_k >= 0 && col_v >= 0 && col_q + H * d <= ld && col_k + H * d <= ld && col_v + H * dv <= ld,
                "lightning attention: columns %d, %d, %d of rows of %d", col_q, col_k, col_v, ld);
     MS_REQUIRE(qkv && decay && state && seq_q_start && seq_q_len && seq_slot && o, "lightning attention: a buffer is missing");
-    const dim3 grid(S, H);
+    MS_REQUIRE(seg_len == 0 || (seg_len % LC == 0 && n_segs > 0 && carry), "lightning attention in chunks: segments of %d need their workspace", seg_len);
     const int dtl = d <= 32 ? 2 : d <= 64 ? 4 : 8, ctl = dv <= 64 ? 1 : 2;
-#define MS_LCH(DTT, CTT)                                                                                                            \
-    hipLaunchKernelGGL((lightning_chunk_kernel<DTT, CTT>), grid, dim3(256),                                                          \
+#define MS_LCH(DTT, CTT, MODE, Z)                                                                                                   \
+    hipLaunchKernelGGL((lightning_chunk_kernel<DTT, CTT>), dim3(S, H, Z), dim3(256),                                                 \
                        sizeof(elem_t) * (2 * LC * DTT * 16 + CTT * 64 * LC + LC * LC) + sizeof(float) * (LC + 1 + 3), stream,       \
-                       (const elem_t*)qkv, ld, col_q, col_k, col_v, decay, state, seq_q_start, seq_q_len, seq_slot, o, H, d, dv)
-    if (dtl == 2 && ctl == 1) MS_LCH(2, 1);
-    else if (dtl == 2) MS_LCH(2, 2);
-    else if (dtl == 4 && ctl == 1) MS_LCH(4, 1);
-    else if (dtl == 4) MS_LCH(4, 2);
-    else if (ctl == 1) MS_LCH(8, 1);
-    else MS_LCH(8, 2);
+                       (const elem_t*)qkv, ld, col_q, col_k, col_v, decay, state, seq_q_start, seq_q_len, seq_slot, o, H, d, dv, MODE, \
+                       seg_len, n_segs, carry)
+#define MS_LCH_ALL(MODE, Z)                                  \
+    do {                                                     \
+        if (dtl == 2 && ctl == 1) MS_LCH(2, 1, MODE, Z);     \
+        else if (dtl == 2) MS_LCH(2, 2, MODE, Z);            \
+        else if (dtl == 4 && ctl == 1) MS_LCH(4, 1, MODE, Z); \
+        else if (dtl == 4) MS_LCH(4, 2, MODE, Z);            \
+        else if (ctl == 1) MS_LCH(8, 1, MODE, Z);            \
+        else MS_LCH(8, 2, MODE, Z);                          \
+    } while (0)
+    if (seg_len == 0) {
+        MS_LCH_ALL(SCAN_WHOLE, 1);
+    } else {
+        MS_LCH_ALL(SCAN_LOCAL, n_segs);
+        if (int rc = check_launch("lightning attention, segments from zero")) return rc;
+        hipLaunchKernelGGL(lightning_carry_kernel, dim3(S, H, ceil_div(d * dv, 256)), dim3(256), 0, stream, decay, state, seq_q_len, seq_slot,
+                           carry, H, d * dv, seg_len, n_segs);
+        if (int rc = check_launch("lightning attention, states between segments")) return rc;
+        MS_LCH_ALL(SCAN_FINAL, n_segs);
+    }
+#undef MS_LCH_ALL
 #undef MS_LCH
     return check_launch("lightning attention in chunks");
 }

@@ -243,7 +243,8 @@ __device__ __forceinline__ void frag_set4(Frag& f, int at, const elem_t* p) {
 }
 
 template <int HPW, int ND, int NT>
-__global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a, const int* __restrict__ seq_q_len, int T) {
+__global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a, const int* __restrict__ seq_q_len, int T, int n_split,
+                                                                     float* __restrict__ part_o, float* __restrict__ part_ml) {
     constexpr int NKS = 4, BK = NT * 16;  // heads of up to 128 numbers
     extern __shared__ float lds[];
     const int H = a.H, d = a.d, dv = a.dv, KV = a.KV, rep = H / KV, ps = a.ps;
@@ -285,7 +286,11 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
         const int* table = a.block_table + (size_t)s * a.table_stride;
         const int a_end = (n_first + BK - 1) / BK;  // tiles of the first tokens: [0, a_end)
         const int b_begin = max(a_end, lo / BK), b_end = p_hi / BK + 1;
-        const int n_tiles = a_end + (b_end - b_begin);
+        const int all_tiles = a_end + (b_end - b_begin);
+        // block (b, y) takes the y-th share of the tiles; the shares are merged by talking_merge_kernel
+        const int per = (all_tiles + n_split - 1) / n_split;
+        const int it_begin = blockIdx.y * per, n_tiles = min(all_tiles, it_begin + per);
+        if (it_begin >= n_tiles) continue;  // the same for every thread of the block
         auto tile_pos = [&](int it) { return (it < a_end ? it : b_begin + (it - a_end)) * BK; };
         auto pages_of = [&](int kt0, int* page) {
 #pragma unroll
@@ -323,10 +328,10 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
         int page[NT], page_n[NT];
         Frag kf[NT][NKS], kf_n[NT][NKS], vf[ND];
         if (active) {
-            pages_of(tile_pos(0), page);
-            load_k(kv0, page, tile_pos(0), kf);
+            pages_of(tile_pos(it_begin), page);
+            load_k(kv0, page, tile_pos(it_begin), kf);
         }
-        for (int it = 0; it < n_tiles; ++it) {
+        for (int it = it_begin; it < n_tiles; ++it) {
             const int kt0 = tile_pos(it);
             if (active) {
                 // this tile's values and the next tile's keys are asked for now and used later
@@ -438,6 +443,21 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
         for (int hh = 0; hh < HPW; ++hh) {
             const int h = h0 + hh;
             if (h >= H) break;
+            if (n_split > 1) {  // this share's maximum, sum and unnormalised output
+                const size_t at = ((size_t)(r0 + r16) * n_split + blockIdx.y) * H + h;
+                if (grp == 0) {
+                    part_ml[2 * at] = m_run[hh];
+                    part_ml[2 * at + 1] = l_run[hh];
+                }
+#pragma unroll
+                for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int e = dt * 16 + grp * 4 + i;
+                        if (e < dv) part_o[at * dv + e] = acc[hh][dt][i];
+                    }
+                continue;
+            }
             const float inv = 1.0f / l_run[hh];
             elem_t* dst = a.out + ((size_t)(r0 + r16) * H + h) * dv;
 #pragma unroll
@@ -619,7 +639,7 @@ __global__ __launch_bounds__(128) void talking_merge_kernel(const float* __restr
         float L = 0.f;
         for (int y = threadIdx.x; y < n_split; y += 64) {
             const float m = ml[(size_t)y * H * 2];
-            const float f = m == -INFINITY ? 0.f : expf(m - M);
+            const float f = (m == -INFINITY || m <= TK_NEG_BIG) ? 0.f : expf(m - M);
             fac[y] = f;
             L += ml[(size_t)y * H * 2 + 1] * f;
         }
@@ -687,19 +707,23 @@ extern "C" int ms_talking_tile_takes(int H, int KV, int d, int dv, int ps) {
 }
 
 template <int HPW, int ND>
-static void launch_tile(const TalkArgs& a, const int* seq_q_len, int T, int NW, hipStream_t stream) {
+static void launch_tile(const TalkArgs& a, const int* seq_q_len, int T, int NW, int n_split, float* part_o, float* part_ml,
+                        hipStream_t stream) {
     const int nt = a.H <= 20 ? 2 : 1;
     const size_t lds = ((size_t)a.H * 16 * nt * 16 + (size_t)a.H * a.H) * sizeof(float);
-    const dim3 grid(ceil_div(T, 16)), block(NW * 64);
-    if (nt == 2) hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 2>), grid, block, lds, stream, a, seq_q_len, T);
-    else hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 1>), grid, block, lds, stream, a, seq_q_len, T);
+    const dim3 grid(ceil_div(T, 16), n_split), block(NW * 64);
+    if (nt == 2)
+        hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 2>), grid, block, lds, stream, a, seq_q_len, T, n_split, part_o, part_ml);
+    else
+        hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 1>), grid, block, lds, stream, a, seq_q_len, T, n_split, part_o, part_ml);
 }
 
 extern "C" int ms_talking_attention_tiles(const void* q, const void* kpool, const void* vpool, const float* talk, const int* block_table,
                                           int table_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, int S,
                                           void* out, int T, int H, int KV, int d, int dv, int ps, int window, int keep_first, float scale,
-                                          hipStream_t stream) {
+                                          int n_split, float* part_o, float* part_ml, hipStream_t stream) {
     MS_REQUIRE(T > 0 && S > 0, "attention: empty problem");
+    MS_REQUIRE(n_split >= 1 && n_split <= 256 && (n_split == 1 || (part_o && part_ml)), "attention in tiles: %d shares", n_split);
     MS_REQUIRE(ms_talking_tile_takes(H, KV, d, dv, ps), "attention in tiles: %d heads over %d, keys of %d, values of %d, pages of %d are not taken",
                H, KV, d, dv, ps);
     MS_REQUIRE(window >= 0 && keep_first >= 0, "attention: window %d, %d first tokens kept", window, keep_first);
@@ -709,7 +733,7 @@ extern "C" int ms_talking_attention_tiles(const void* q, const void* kpool, cons
     TalkArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, talk, block_table, table_stride, seq_q_start, seq_pos0,
                S, (elem_t*)out, H, KV, d, dv, ps, window, keep_first, scale};
     const int hpw = H <= 8 ? 1 : H <= 16 ? 2 : 4, nw = ceil_div(H, hpw), nd = ceil_div(dv, 16);
-#define MS_TILE(HP, NDD) launch_tile<HP, NDD>(a, seq_q_len, T, nw, stream)
+#define MS_TILE(HP, NDD) launch_tile<HP, NDD>(a, seq_q_len, T, nw, n_split, part_o, part_ml, stream)
 #define MS_TILE_ND(HP)                      \
     do {                                    \
         if (nd <= 1) MS_TILE(HP, 1);        \
@@ -722,7 +746,12 @@ extern "C" int ms_talking_attention_tiles(const void* q, const void* kpool, cons
     else MS_TILE_ND(4);
 #undef MS_TILE_ND
 #undef MS_TILE
-    return check_launch("attention in tiles");
+    if (int rc = check_launch("attention in tiles")) return rc;
+    if (n_split > 1) {
+        hipLaunchKernelGGL(talking_merge_kernel, dim3(T, H), dim3(128), 0, stream, part_o, part_ml, (elem_t*)out, n_split, H, dv);
+        return check_launch("attention merge");
+    }
+    return 0;
 }
 
 // Whether the kernel whose blocks share a row's keys takes these sizes (else: one block a row, element by element).

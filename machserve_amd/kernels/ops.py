@@ -640,6 +640,8 @@ class HipOps:
                                                self._stream()))
         return y
 
+    LIGHTNING_SEGMENT = 128  # rows of a segment of lightning attention in chunks (a multiple of the chunk of 32)
+
     def lightning_attention(self, qkvg: torch.Tensor, heads: int, dim: int, vdim: int, decay: torch.Tensor, state: torch.Tensor,
                             seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_slot: torch.Tensor, chunked: bool = False) -> torch.Tensor:
         """Linear attention with a decay per head over the step's rows.  ``qkvg [T, ld]`` holds q ``[heads, dim]``, k
@@ -653,8 +655,22 @@ class HipOps:
         self._want(state, torch.float32, "lightning state", state.shape[0], heads, dim, vdim)
         S = self._seq_operands("lightning", seq_q_start, seq_q_len, seq_slot)
         o = torch.empty((T, heads * vdim), dtype=torch.float32, device=qkvg.device)
-        fn = lib.ms_lightning_chunked if chunked and self._plan("ms_lightning_chunked_takes", dim, vdim, lib=lib) else lib.ms_lightning
-        self._check(lib, fn(_ptr(qkvg), _c_int(ld), _c_int(0), _c_int(heads * dim), _c_int(2 * heads * dim), _ptr(decay),
+        if chunked and self._plan("ms_lightning_chunked_takes", dim, vdim, lib=lib):
+            # long portions in segments that are walked side by side (see selective_scan); the cut follows from the step's
+            # rows and requests alone
+            seg = n_segs = 0
+            carry = None
+            if T >= 2 * self.LIGHTNING_SEGMENT and T // S >= self.LIGHTNING_SEGMENT:
+                n_segs = -(-T // self.LIGHTNING_SEGMENT)
+                if S * n_segs * heads * dim * vdim * 4 <= (256 << 20):
+                    seg = self.LIGHTNING_SEGMENT
+                    carry = torch.empty((S, n_segs, heads, dim, vdim), dtype=torch.float32, device=qkvg.device)
+            self._check(lib, lib.ms_lightning_chunked(
+                _ptr(qkvg), _c_int(ld), _c_int(0), _c_int(heads * dim), _c_int(2 * heads * dim), _ptr(decay), _ptr(state), _ptr(seq_q_start),
+                _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(o), _c_int(T), _c_int(heads), _c_int(dim), _c_int(vdim), _c_int(seg),
+                _c_int(n_segs if seg else 0), _ptr(carry), self._stream()))
+            return o
+        self._check(lib, lib.ms_lightning(_ptr(qkvg), _c_int(ld), _c_int(0), _c_int(heads * dim), _c_int(2 * heads * dim), _ptr(decay),
                                           _ptr(state), _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(o),
                                           _c_int(T), _c_int(heads), _c_int(dim), _c_int(vdim), self._stream()))
         return o
@@ -747,10 +763,19 @@ class HipOps:
         out = torch.empty((T, H * dv), dtype=self.dtype, device=q.device)
         if tiles and self.talking_tile_takes(H, KV, d, dv, page_size):
             self._want(seq_q_len, torch.int32, "seq_q_len", S)
+            # too few tiles of rows to fill the chip: several blocks share a tile's keys (at least four 32-key tiles each)
+            span = block_table.shape[1] * page_size
+            key_tiles = -(-span // 32) if not window else min(-(-span // 32), -(-window // 32) + 2 + -(-keep_first // 32))
+            n_split = max(1, min(8, (2 * self._cus) // -(-T // 16), key_tiles // 4))
+            part_o = part_ml = None
+            if n_split > 1:
+                part_o = torch.empty((T, n_split, H * dv), dtype=torch.float32, device=q.device)
+                part_ml = torch.empty((T, n_split, H, 2), dtype=torch.float32, device=q.device)
             self._check(lib, lib.ms_talking_attention_tiles(
                 _ptr(q), _ptr(kpool), _ptr(vpool), _ptr(talk), _ptr(block_table), _c_int(block_table.shape[1]), _ptr(seq_q_start),
                 _ptr(seq_q_len), _ptr(seq_pos0), _c_int(S), _ptr(out), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv),
-                _c_int(page_size), _c_int(window or 0), _c_int(keep_first), _c_float(scale), self._stream()))
+                _c_int(page_size), _c_int(window or 0), _c_int(keep_first), _c_float(scale), _c_int(n_split), _ptr(part_o), _ptr(part_ml),
+                self._stream()))
             return out
         if self._plan("ms_talking_split_takes", H, KV, d, dv, page_size, lib=lib):
             # blocks that share a row's keys, as many as fill the chip: how many follows from the step's rows and the
