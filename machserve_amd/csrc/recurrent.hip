@@ -68,8 +68,9 @@ __global__ __launch_bounds__(256) void conv_state_kernel(const elem_t* __restric
 // ---- step sizes ------------------------------------------------------------------------
 // dt[t, c] = softplus(b[c] + sum_r wt[r, c] * low[t, r]), low = the first R columns of the rows of `dbc`; `wt` is the
 // projection transposed, [R, C], so that the threads of a wave read neighbouring numbers.  A block takes DT_ROWS rows
-// and 256 channels: a weight is read once for all of its rows.
-constexpr int DT_ROWS = 8;
+// and 256 channels: a weight is read once for all of its rows (eight in steps of many rows, one where rows are few and
+// the blocks would not fill the chip).
+template <int DT_ROWS>
 __global__ __launch_bounds__(256) void dt_softplus_kernel(const float* __restrict__ dbc, int ldb, const float* __restrict__ wt,
                                                           const float* __restrict__ b, float* __restrict__ dt, int T, int C, int R) {
     extern __shared__ float low[];  // [DT_ROWS][R]
@@ -193,6 +194,78 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(const elem_t* __res
 #pragma unroll
         for (int k = 0; k < SPL; ++k)
             if (ns[k] >= 0) st[ns[k]] = S[k];
+    }
+}
+
+// The chunks of a long portion are many, so there a thread takes a whole channel, its states in registers: no sum over
+// lanes, and what belongs to the channel (step size, input, gate) is worked out once, not once a state.
+constexpr int WIDE_TILE = 8;
+template <int NMAX>
+__global__ __launch_bounds__(64) void selective_scan_wide_kernel(const elem_t* __restrict__ x, const elem_t* __restrict__ z, int ldz,
+                                                                 const float* __restrict__ dt, const float* __restrict__ dbc, int ldb,
+                                                                 int col_b, int col_c, const float* __restrict__ a_log,
+                                                                 const float* __restrict__ dskip, float* __restrict__ state,
+                                                                 const int* __restrict__ seq_q_start, const int* __restrict__ seq_q_len,
+                                                                 const int* __restrict__ seq_slot, elem_t* __restrict__ y, int C, int N,
+                                                                 int mode, int chunk_len, int n_chunks, float* __restrict__ carry,
+                                                                 float* __restrict__ csum) {
+    const int s = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+    const int left = seq_q_len[s] - blockIdx.z * chunk_len;
+    if (left <= 0) return;
+    const int q0 = seq_q_start[s] + blockIdx.z * chunk_len, n_rows = min(left, chunk_len);
+    const bool last = n_rows == left;
+    if ((mode == SCAN_LOCAL && last) || c >= C) return;
+    float* pass = carry + (((size_t)s * n_chunks + blockIdx.z) * C + c) * N;
+    float S[NMAX], A[NMAX];
+#pragma unroll
+    for (int n = 0; n < NMAX; ++n) {
+        S[n] = (n < N && mode != SCAN_LOCAL) ? pass[n] : 0.f;
+        A[n] = n < N ? -expf(a_log[(size_t)c * N + n]) : 0.f;
+    }
+    const float dsk = dskip ? dskip[c] : 0.f;
+    float dsum = 0.f;
+    for (int i0 = 0; i0 < n_rows; i0 += WIDE_TILE) {
+        float d[WIDE_TILE], xv[WIDE_TILE], zv[WIDE_TILE];
+#pragma unroll
+        for (int j = 0; j < WIDE_TILE; ++j) {  // a tile's numbers at once
+            const size_t t = (size_t)(q0 + min(i0 + j, n_rows - 1));
+            d[j] = dt[t * C + c];
+            xv[j] = to_f32(x[t * C + c]);
+            zv[j] = mode == SCAN_LOCAL ? 0.f : to_f32(z[t * ldz + c]);
+        }
+#pragma unroll
+        for (int j = 0; j < WIDE_TILE; ++j) {
+            if (i0 + j < n_rows) {
+                const float* Bt = dbc + (size_t)(q0 + i0 + j) * ldb + col_b;
+                const float* Ct = dbc + (size_t)(q0 + i0 + j) * ldb + col_c;
+                const float dx = d[j] * xv[j];
+                dsum += d[j];
+                float acc = 0.f;
+#pragma unroll
+                for (int n = 0; n < NMAX; ++n) {
+                    if (n < N) {
+#ifdef MS_ELEM_HALF
+                        S[n] = __expf(d[j] * A[n]) * S[n] + dx * Bt[n];
+#else
+                        S[n] = expf(d[j] * A[n]) * S[n] + dx * Bt[n];
+#endif
+                        acc += S[n] * Ct[n];
+                    }
+                }
+                if (mode != SCAN_LOCAL) y[(size_t)(q0 + i0 + j) * C + c] = from_f32<elem_t>((acc + dsk * xv[j]) * silu_f(zv[j]));
+            }
+        }
+    }
+    if (mode == SCAN_LOCAL) {
+#pragma unroll
+        for (int n = 0; n < NMAX; ++n)
+            if (n < N) pass[n] = S[n];
+        csum[((size_t)s * n_chunks + blockIdx.z) * C + c] = dsum;
+    } else if (last) {
+        float* st = state + ((size_t)seq_slot[s] * C + c) * N;
+#pragma unroll
+        for (int n = 0; n < NMAX; ++n)
+            if (n < N) st[n] = S[n];
     }
 }
 
@@ -530,9 +603,13 @@ extern "C" int ms_dt_softplus(const float* dbc, int ldb, const float* w, const f
                               hipStream_t stream) {
     MS_REQUIRE(T > 0 && C > 0 && R > 0 && ldb >= R, "step sizes: T=%d C=%d R=%d ld=%d", T, C, R, ldb);
     MS_REQUIRE(dbc && w && dt, "step sizes: a buffer is missing");
-    MS_REQUIRE((size_t)DT_ROWS * R * sizeof(float) <= 48 * 1024, "step sizes: a bottleneck of %d is too wide", R);
-    hipLaunchKernelGGL(dt_softplus_kernel, dim3(ceil_div(T, DT_ROWS), ceil_div(C, 256)), dim3(256), (size_t)DT_ROWS * R * sizeof(float), stream,
-                       dbc, ldb, w, b, dt, T, C, R);
+    MS_REQUIRE((size_t)8 * R * sizeof(float) <= 48 * 1024, "step sizes: a bottleneck of %d is too wide", R);
+    if (T >= 128)
+        hipLaunchKernelGGL(dt_softplus_kernel<8>, dim3(ceil_div(T, 8), ceil_div(C, 256)), dim3(256), (size_t)8 * R * sizeof(float), stream, dbc,
+                           ldb, w, b, dt, T, C, R);
+    else
+        hipLaunchKernelGGL(dt_softplus_kernel<1>, dim3(T, ceil_div(C, 256)), dim3(256), (size_t)R * sizeof(float), stream, dbc, ldb, w, b, dt,
+                           T, C, R);
     return check_launch("step sizes");
 }
 
@@ -558,6 +635,20 @@ extern "C" int ms_selective_scan(const void* x, const void* z, int ldz, const fl
     } while (0)
     if (chunk_len == 0) {
         MS_SCAN_N(SCAN_WHOLE, 1);
+    } else if (N <= 32) {  // a channel a thread, its states in registers
+#define MS_WIDE(NM, MODE)                                                                                                          \
+    hipLaunchKernelGGL(selective_scan_wide_kernel<NM>, dim3(S, ceil_div(C, 64), n_chunks), dim3(64), 0, stream, (const elem_t*)x,    \
+                       (const elem_t*)z, ldz, dt, dbc, ldb, col_b, col_c, a_log, dskip, state, seq_q_start, seq_q_len, seq_slot,     \
+                       (elem_t*)y, C, N, MODE, chunk_len, n_chunks, carry, csum)
+        if (N <= 16) MS_WIDE(16, SCAN_LOCAL);
+        else MS_WIDE(32, SCAN_LOCAL);
+        if (int rc = check_launch("selective scan, chunks from zero")) return rc;
+        hipLaunchKernelGGL(scan_carry_kernel, dim3(S, (unsigned)ceil_div((long)C * N, 256L)), dim3(256), 0, stream, a_log, state, seq_q_len,
+                           seq_slot, carry, csum, C, N, chunk_len, n_chunks);
+        if (int rc = check_launch("selective scan, states between chunks")) return rc;
+        if (N <= 16) MS_WIDE(16, SCAN_FINAL);
+        else MS_WIDE(32, SCAN_FINAL);
+#undef MS_WIDE
     } else {
         MS_SCAN_N(SCAN_LOCAL, n_chunks);
         if (int rc = check_launch("selective scan, chunks from zero")) return rc;

@@ -140,11 +140,12 @@ def test_long_lightning_attention_in_segments_equals_the_walk_token_after_token(
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_a_long_scan_in_chunks_equals_the_walk_token_after_token(dtype):
+@pytest.mark.parametrize("C,N", [(48, 12), (70, 24), (33, 40)])
+def test_a_long_scan_in_chunks_equals_the_walk_token_after_token(dtype, C, N):
     """Steps of many rows cut their requests into chunks that are walked side by side; the result is the one walk's."""
     ops = ops_of(dtype)
     torch.manual_seed(5)
-    C, N, R, lens = 48, 12, 3, [300, 1, 129, 210]
+    R, lens = 3, [300, 1, 129, 210]
     T = sum(lens)
     assert T >= ops.SCAN_CHUNK_MIN_ROWS and T // len(lens) >= ops.SCAN_CHUNK_MIN_ROWS // 2
     x, z = (torch.randn(T, C).to(dtype).float() for _ in range(2))
