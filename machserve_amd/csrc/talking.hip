@@ -495,7 +495,10 @@ __global__ __launch_bounds__(256) void talking_attention_split_kernel(TalkArgs a
     float* head_l = head_m + H;
     float* head_a = head_l + H;
     int* page_of = reinterpret_cast<int*>(head_a + H);  // [4] pages of the tile's 16-position parts, -1: none
+    float* talk_s = reinterpret_cast<float*>(page_of + 4);  // [H][H]
     const int t = blockIdx.x, y = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (a.talk)
+        for (int i = tid; i < H * H; i += 256) talk_s[i] = a.talk[i];
     const int s = seq_of_row(t, a.seq_q_start, a.S);
     const int pos = a.seq_pos0[s] + (t - a.seq_q_start[s]);
     const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
@@ -531,15 +534,25 @@ __global__ __launch_bounds__(256) void talking_attention_split_kernel(TalkArgs a
             for (int r = 0; r < TK_MAX_REP; ++r) sc[r] = 0.f;
             if (page >= 0 && key <= pos) {
                 const elem_t* kr = a.kpool + (((size_t)page * KV + kvh) * ps + key % ps) * d;
-                for (int c8 = 0; c8 < d; c8 += 8) {
-                    float k8[8];
-                    load8(kr + c8, k8);
+                for (int c0 = 0; c0 < d; c0 += 128) {  // 128 numbers of the key's row are asked for at once
+                    Frag kf[16];
 #pragma unroll
-                    for (int r = 0; r < TK_MAX_REP; ++r) {
-                        if (r < rep) {
-                            const float* qr = qs + (kvh * rep + r) * d + c8;
+                    for (int c = 0; c < 16; ++c)
+                        if (c0 + c * 8 < d) kf[c] = frag_load(kr + c0 + c * 8);
 #pragma unroll
-                            for (int e = 0; e < 8; ++e) sc[r] += qr[e] * k8[e];
+                    for (int c = 0; c < 16; ++c) {
+                        if (c0 + c * 8 < d) {
+                            float k8[8];
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) k8[e] = to_f32(kf[c].v[e]);
+#pragma unroll
+                            for (int r = 0; r < TK_MAX_REP; ++r) {
+                                if (r < rep) {
+                                    const float* qr = qs + (kvh * rep + r) * d + c0 + c * 8;
+#pragma unroll
+                                    for (int e = 0; e < 8; ++e) sc[r] += qr[e] * k8[e];
+                                }
+                            }
                         }
                     }
                 }
@@ -554,7 +567,7 @@ __global__ __launch_bounds__(256) void talking_attention_split_kernel(TalkArgs a
             float sc;
             if (a.talk) {
                 sc = 0.f;
-                for (int g = 0; g < H; ++g) sc += a.talk[h * H + g] * raw[g * TK_KEYS + jj];
+                for (int g = 0; g < H; ++g) sc += talk_s[h * H + g] * raw[g * TK_KEYS + jj];
             } else {
                 sc = raw[item];
             }
@@ -583,20 +596,19 @@ __global__ __launch_bounds__(256) void talking_attention_split_kernel(TalkArgs a
             if (c < n_out) {
                 const int h = c / dv, e = c - h * dv, kvh = h / rep;
                 float sum = 0.f;
+                Frag vf[8];  // the tile's 64 values of this column: asked for at once
 #pragma unroll
                 for (int sub = 0; sub < 4; ++sub) {
-                    const int page = page_of[sub];
-                    if (page < 0) continue;
+                    const int page = max(page_of[sub], 0);
                     const elem_t* vr = a.vpool + (((size_t)page * KV + kvh) * dv + e) * ps + (kt0 + sub * 16) % ps;
-                    const float* w = mix + h * TK_KEYS + sub * 16;
-                    float v8[8];
-                    load8(vr, v8);
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) sum += w[k] * v8[k];
-                    load8(vr + 8, v8);
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) sum += w[8 + k] * v8[k];
+                    vf[2 * sub] = frag_load(vr);
+                    vf[2 * sub + 1] = frag_load(vr + 8);
                 }
+                const float* w = mix + h * TK_KEYS;  // a weight of a part without a page is zero
+#pragma unroll
+                for (int f = 0; f < 8; ++f)
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) sum += w[f * 8 + k] * to_f32(vf[f].v[k]);
                 acc[i] = acc[i] * head_a[h] + sum;
             }
         }
@@ -757,7 +769,7 @@ extern "C" int ms_talking_attention_tiles(const void* q, const void* kpool, cons
 // Whether the kernel whose blocks share a row's keys takes these sizes (else: one block a row, element by element).
 extern "C" int ms_talking_split_takes(int H, int KV, int d, int dv, int ps) {
     if (H < 1 || KV < 1 || H % KV || H / KV > TK_MAX_REP || d % 8 || ps % 16 || H * dv > 256 * TK_MAX_OUT) return 0;
-    return ((size_t)H * d + 2 * (size_t)H * TK_KEYS + 3 * (size_t)H + 4) * sizeof(float) <= (size_t)TK_MAX_LDS;
+    return ((size_t)H * d + 2 * (size_t)H * TK_KEYS + 3 * (size_t)H + 4 + (size_t)H * H) * sizeof(float) <= (size_t)TK_MAX_LDS;
 }
 
 // part_o float [T, n_split, H * dv] and part_ml float [T, n_split, H, 2] are the shares' workspace (unused with one share).
@@ -775,7 +787,7 @@ extern "C" int ms_talking_attention_split(const void* q, const void* kpool, cons
                "attention in shares: operands must be 16-byte aligned");
     TalkArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, talk, block_table, table_stride, seq_q_start, seq_pos0,
                S, (elem_t*)out, H, KV, d, dv, ps, window, keep_first, scale};
-    const size_t lds = ((size_t)H * d + 2 * (size_t)H * TK_KEYS + 3 * (size_t)H + 4) * sizeof(float);
+    const size_t lds = ((size_t)H * d + 2 * (size_t)H * TK_KEYS + 3 * (size_t)H + 4 + (size_t)H * H) * sizeof(float);
     hipLaunchKernelGGL(talking_attention_split_kernel, dim3(T, n_split), dim3(256), lds, stream, a, n_split, part_o, part_ml);
     if (int rc = check_launch("attention in shares")) return rc;
     if (n_split > 1) {

@@ -52,8 +52,9 @@ class TalkingAttention(Mixer):
         return decls
 
     def ignored_tensors(self):
-        """The layer whose values the others blend with has a blend weight in the checkpoint that nothing reads."""
-        return [self.spec.tensors.get("blend", "blend")] if self.spec.value_blend == "source" else []
+        """A layer that does not blend (the one whose values the others blend with, or one outside the blending) may
+        have a blend weight in the checkpoint that nothing reads."""
+        return [self.spec.tensors.get("blend", "blend")] if self.spec.value_blend != "blend" else []
 
     def load(self, t):
         self.w_qkv = torch.cat([t["q.weight"], t["k.weight"], t["v.weight"]], dim=0).contiguous()
@@ -87,8 +88,9 @@ class TalkingAttention(Mixer):
                                      view.page_size)
         if s.value_blend == "source":
             ctx.shared[shared] = own
-        # a step of many rows runs in tiles of 16 rows on the matrix cores, single decoded rows one row a block
-        tiles = not ctx.decode_only and ctx.n_rows >= getattr(ops, "TILE_MIN_ROWS", 1 << 30)
+        # a step of many rows a request runs in tiles of 16 rows on the matrix cores, single decoded rows (and steps that
+        # are mostly such rows: a tile takes its requests one after the other) one row a block
+        tiles = not ctx.decode_only and ctx.n_rows >= max(getattr(ops, "TILE_MIN_ROWS", 1 << 30), 4 * ctx.n_seqs)
         o = ops.talking_attention(q, self.kpool, self.vpool, self.talk, view.block_table, ctx.seq_q_start, ctx.seq_pos0, s.heads,
                                   s.kv_heads, s.head_dim, s.v_head_dim, view.page_size, s.window, s.keep_first, float(s.scale),
                                   ctx.seq_q_len, tiles)
