@@ -57,7 +57,7 @@ class AttentionLayer:
     dim: int
     vdim: int
     scale: float
-    window: int
+    window: Optional[int]
     keep_first: int
     rot: RotationConfig
     v_mix: bool
@@ -88,8 +88,8 @@ def _mixer_of(kind: str, m: dict, where: str):
         if heads % kv:
             raise ConfigError(f"config.json: '{where}heads' {heads} is not a multiple of '{where}kv_heads' {kv}")
         dim = _int(m, "dim", where)
-        mask = _get(m, "mask", where)
-        rot = _get(m, "rot", where)
+        mask = m.get("mask")  # none: every earlier token is seen
+        rot = m.get("rot") or {"dims": 0, "base": 10000.0}  # none: nothing is rotated
         dims = _int(rot, "dims", where + "rot.", 0)
         if dims % 2 or dims > dim:
             raise ConfigError(f"config.json: '{where}rot.dims' {dims} must be even and at most '{where}dim' {dim}")
@@ -97,9 +97,10 @@ def _mixer_of(kind: str, m: dict, where: str):
         scaling = None
         if sc is not None:
             w = where + "rot.scaling."
-            scaling = (_num(sc, "factor", w), _int(sc, "original", w), _num(sc, "fast", w), _num(sc, "slow", w))
-        return AttentionLayer(heads, kv, dim, _int(m, "vdim", where), _num(m, "scale", where), _int(mask, "size", where + "mask."),
-                              _int(mask, "keep_first", where + "mask.", 0),
+            scaling = (_num(sc, "factor", w), int(_num(sc, "original", w)), _num(sc, "fast", w), _num(sc, "slow", w))
+        return AttentionLayer(heads, kv, dim, _int(m, "vdim", where), _num(m, "scale", where),
+                              _int(mask, "size", where + "mask.") if mask is not None else None,
+                              _int(mask, "keep_first", where + "mask.", 0) if mask is not None and mask.get("keep_first") is not None else 0,
                               RotationConfig(_num(rot, "base", where + "rot."), dims, scaling), bool(m.get("v_mix", False)))
     if kind == "mamba1":
         return Mamba1Layer(_int(m, "inner", where), _int(m, "state", where), _int(m, "dt_rank", where), _int(m, "conv", where))
@@ -158,8 +159,9 @@ class RenanexConfig:
                 if m.rot.scaling is not None:
                     f, o, fast, slow = m.rot.scaling
                     rot["scaling"] = {"factor": f, "original": o, "fast": fast, "slow": slow}
-                mixer = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim, "scale": m.scale,
-                         "mask": {"size": m.window, "keep_first": m.keep_first}, "rot": rot, "v_mix": m.v_mix}
+                mixer = {"heads": m.heads, "kv_heads": m.kv_heads, "dim": m.dim, "vdim": m.vdim, "scale": m.scale, "rot": rot, "v_mix": m.v_mix}
+                if m.window is not None:
+                    mixer["mask"] = {"size": m.window, "keep_first": m.keep_first}
             elif isinstance(m, Mamba1Layer):
                 mixer = {"inner": m.inner, "state": m.state, "dt_rank": m.dt_rank, "conv": m.conv}
             else:
