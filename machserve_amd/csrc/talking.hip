@@ -231,6 +231,16 @@ __global__ __launch_bounds__(256) void talking_attention_kernel(TalkArgs a) {
 // taken request by request: the rows of the others are masked, which leaves their sums as they are.
 constexpr float TK_NEG_BIG = -1.0e30f;
 
+// e^x for the softmax of the tile kernel: the hardware's exponential in the two-byte builds (a few units in the last
+// place of 32 bits, far below the rounding of the weights to the element type as operands), the library's in 32-bit
+__device__ __forceinline__ float tk_exp(float x) {
+#ifdef MS_ELEM_HALF
+    return __expf(x);
+#else
+    return expf(x);
+#endif
+}
+
 // 4 or 8 elements of one row that lie side by side, into elements at .. of a fragment
 __device__ __forceinline__ void frag_set4(Frag& f, int at, const elem_t* p) {
 #ifdef MS_ELEM_HALF
@@ -405,13 +415,15 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
                     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            const float p = ok[nt][i] ? expf(mixed[nt][i] - m_new) : 0.f;
+                            const float p = ok[nt][i] ? tk_exp(mixed[nt][i] - m_new) : 0.f;
                             mixed[nt][i] = p;
                             psum += p;
                         }
                     psum += __shfl_xor(psum, 16, WAVE);
                     psum += __shfl_xor(psum, 32, WAVE);
-                    const float alpha = expf(m_run[hh] - m_new);
+                    // where no row's maximum rose the factor is exactly one: after the first tiles that is the rule
+                    const bool rose = __any(m_new > m_run[hh]);
+                    const float alpha = rose ? tk_exp(m_run[hh] - m_new) : 1.0f;
                     l_run[hh] = l_run[hh] * alpha + psum;
                     m_run[hh] = m_new;
                     Frag pf;
@@ -420,12 +432,14 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
                         pf.v[i] = from_f32<elem_t>(mixed[0][i]);
                         pf.v[4 + i] = from_f32<elem_t>(NT > 1 ? mixed[NT - 1][i] : 0.f);
                     }
+                    if (rose) {
 #pragma unroll
-                    for (int dt = 0; dt < ND; ++dt) {
+                        for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) acc[hh][dt][i] *= alpha;
-                        mma_16x16x32(acc[hh][dt], vf[dt], pf);
+                            for (int i = 0; i < 4; ++i) acc[hh][dt][i] *= alpha;
                     }
+#pragma unroll
+                    for (int dt = 0; dt < ND; ++dt) mma_16x16x32(acc[hh][dt], vf[dt], pf);
                 }
             }
             __syncthreads();
