@@ -254,15 +254,19 @@ __device__ __forceinline__ void frag_set4(Frag& f, int at, const elem_t* p) {
 
 template <int HPW, int ND, int NT>
 __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a, const int* __restrict__ seq_q_len, int T, int n_split,
-                                                                     float* __restrict__ part_o, float* __restrict__ part_ml) {
+                                                                     float* __restrict__ part_o, float* __restrict__ part_ml, int tile_rows) {
     constexpr int NKS = 4, BK = NT * 16;  // heads of up to 128 numbers
     extern __shared__ float lds[];
     const int H = a.H, d = a.d, dv = a.dv, KV = a.KV, rep = H / KV, ps = a.ps;
-    float* raw = lds;                                // [H][16 queries][NT * 16 keys]
+    // [H][NT][64 lanes][4]: a lane reads what the same lane of the wave that owns head g wrote (both hold the same
+    // (key, query) pairs), so a wave's 64 lanes always touch 1,024 consecutive bytes: no two of them meet in a bank
+    float* raw = lds;
     float* talk_s = raw + (size_t)H * 16 * NT * 16;  // [H][H]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r16 = lane & 15, grp = lane >> 4;
-    const int r0 = blockIdx.x * 16, r_end = min(r0 + 16, T);
-    const int my_row = min(r0 + r16, T - 1);
+    // tile_rows = 16: a tile of the step's rows; 1: one row a block, the tile's other fifteen queries idle (decoding: the
+    // rows belong to different requests, which a tile would take one after the other)
+    const int r0 = blockIdx.x * tile_rows, r_end = min(r0 + tile_rows, T);
+    const int my_row = min(r0 + r16, r_end - 1);
     const int h0 = wave * HPW;
     const bool active = h0 < H;  // a wave beyond the heads only keeps the barriers
     if (a.talk)
@@ -366,7 +370,7 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
 #pragma unroll
                         for (int ks = 0; ks < NKS; ++ks)
                             if (ks * 32 < d) mma_16x16x32(sc, kf[nt][ks], qf[hh][ks]);
-                        *reinterpret_cast<f32x4*>(raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4) = sc * a.scale;
+                        *reinterpret_cast<f32x4*>(raw + (((size_t)h * NT + nt) * 64 + lane) * 4) = sc * a.scale;
                     }
                 }
             }
@@ -390,12 +394,12 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
                             const float w = talk_s[h * H + g];
 #pragma unroll
                             for (int nt = 0; nt < NT; ++nt)
-                                mixed[nt] += w * *reinterpret_cast<const f32x4*>(raw + (((size_t)g * 16 + r16) * NT + nt) * 16 + grp * 4);
+                                mixed[nt] += w * *reinterpret_cast<const f32x4*>(raw + (((size_t)g * NT + nt) * 64 + lane) * 4);
                         }
                     } else {
 #pragma unroll
                         for (int nt = 0; nt < NT; ++nt)
-                            mixed[nt] = *reinterpret_cast<const f32x4*>(raw + (((size_t)h * 16 + r16) * NT + nt) * 16 + grp * 4);
+                            mixed[nt] = *reinterpret_cast<const f32x4*>(raw + (((size_t)h * NT + nt) * 64 + lane) * 4);
                     }
                     bool ok[NT][4];
                     float tmax = TK_NEG_BIG;
@@ -452,7 +456,7 @@ __global__ __launch_bounds__(512) void talking_attention_tile_kernel(TalkArgs a,
         }
     }
     // O^T: lane holds value columns dt * 16 + grp * 4 + i of query r16
-    if (r0 + r16 < T && active) {
+    if (r0 + r16 < r_end && active) {
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
             const int h = h0 + hh;
@@ -733,22 +737,25 @@ extern "C" int ms_talking_tile_takes(int H, int KV, int d, int dv, int ps) {
 }
 
 template <int HPW, int ND>
-static void launch_tile(const TalkArgs& a, const int* seq_q_len, int T, int NW, int n_split, float* part_o, float* part_ml,
+static void launch_tile(const TalkArgs& a, const int* seq_q_len, int T, int NW, int n_split, float* part_o, float* part_ml, int tile_rows,
                         hipStream_t stream) {
     const int nt = a.H <= 20 ? 2 : 1;
     const size_t lds = ((size_t)a.H * 16 * nt * 16 + (size_t)a.H * a.H) * sizeof(float);
-    const dim3 grid(ceil_div(T, 16), n_split), block(NW * 64);
+    const dim3 grid(ceil_div(T, tile_rows), n_split), block(NW * 64);
     if (nt == 2)
-        hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 2>), grid, block, lds, stream, a, seq_q_len, T, n_split, part_o, part_ml);
+        hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 2>), grid, block, lds, stream, a, seq_q_len, T, n_split, part_o, part_ml,
+                           tile_rows);
     else
-        hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 1>), grid, block, lds, stream, a, seq_q_len, T, n_split, part_o, part_ml);
+        hipLaunchKernelGGL((talking_attention_tile_kernel<HPW, ND, 1>), grid, block, lds, stream, a, seq_q_len, T, n_split, part_o, part_ml,
+                           tile_rows);
 }
 
 extern "C" int ms_talking_attention_tiles(const void* q, const void* kpool, const void* vpool, const float* talk, const int* block_table,
                                           int table_stride, const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, int S,
                                           void* out, int T, int H, int KV, int d, int dv, int ps, int window, int keep_first, float scale,
-                                          int n_split, float* part_o, float* part_ml, hipStream_t stream) {
+                                          int n_split, float* part_o, float* part_ml, int tile_rows, hipStream_t stream) {
     MS_REQUIRE(T > 0 && S > 0, "attention: empty problem");
+    MS_REQUIRE(tile_rows == 16 || tile_rows == 1, "attention in tiles: tiles of %d rows", tile_rows);
     MS_REQUIRE(n_split >= 1 && n_split <= 256 && (n_split == 1 || (part_o && part_ml)), "attention in tiles: %d shares", n_split);
     MS_REQUIRE(ms_talking_tile_takes(H, KV, d, dv, ps), "attention in tiles: %d heads over %d, keys of %d, values of %d, pages of %d are not taken",
                H, KV, d, dv, ps);
@@ -759,7 +766,7 @@ extern "C" int ms_talking_attention_tiles(const void* q, const void* kpool, cons
     TalkArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, talk, block_table, table_stride, seq_q_start, seq_pos0,
                S, (elem_t*)out, H, KV, d, dv, ps, window, keep_first, scale};
     const int hpw = H <= 8 ? 1 : H <= 16 ? 2 : 4, nw = ceil_div(H, hpw), nd = ceil_div(dv, 16);
-#define MS_TILE(HP, NDD) launch_tile<HP, NDD>(a, seq_q_len, T, nw, n_split, part_o, part_ml, stream)
+#define MS_TILE(HP, NDD) launch_tile<HP, NDD>(a, seq_q_len, T, nw, n_split, part_o, part_ml, tile_rows, stream)
 #define MS_TILE_ND(HP)                      \
     do {                                    \
         if (nd <= 1) MS_TILE(HP, 1);        \

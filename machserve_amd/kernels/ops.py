@@ -744,8 +744,9 @@ class HipOps:
                           seq_q_len: Optional[torch.Tensor] = None, tiles: bool = False) -> torch.Tensor:
         """Attention of every row over the keys it sees: the last ``window`` positions up to its own (None: all) and
         the request's first ``keep_first``.  ``talk`` float32 ``[H, H]`` mixes the heads' scaled scores before the
-        softmax (None: no exchange).  Returns ``[T, H * dv]`` in the element type.  ``tiles`` (with ``seq_q_len``): 16
-        rows a block on the matrix cores, for steps of many rows; else one row a block, for decoding."""
+        softmax (None: no exchange).  Returns ``[T, H * dv]`` in the element type.  ``tiles``: 16 rows a block, for steps
+        of many rows a request; else one row a block, for decoding.  With ``seq_q_len`` and sizes it takes, the kernel on
+        the matrix cores runs either way; else the kernels of the vector units (one row a block)."""
         lib = self._extra_lib("talking")
         T = q.shape[0]
         self._want(q, self.dtype, "attention q", T, H * d)
@@ -761,12 +762,15 @@ class HipOps:
         self._want(seq_q_start, torch.int32, "seq_q_start", S)
         self._want(seq_pos0, torch.int32, "seq_pos0", S)
         out = torch.empty((T, H * dv), dtype=self.dtype, device=q.device)
-        if tiles and self.talking_tile_takes(H, KV, d, dv, page_size):
+        if self.talking_tile_takes(H, KV, d, dv, page_size) and seq_q_len is not None:
+            # On the matrix cores: tiles of 16 rows for steps of many rows a request; for single decoded rows a block a
+            # row (a tile with one live query: the rows belong to different requests, which a tile takes one after the
+            # other).  Too few tiles to fill the chip: several blocks share a tile's keys (at least four 32-key tiles each).
             self._want(seq_q_len, torch.int32, "seq_q_len", S)
-            # too few tiles of rows to fill the chip: several blocks share a tile's keys (at least four 32-key tiles each)
+            tile_rows = 16 if tiles else 1
             span = block_table.shape[1] * page_size
             key_tiles = -(-span // 32) if not window else min(-(-span // 32), -(-window // 32) + 2 + -(-keep_first // 32))
-            n_split = max(1, min(8, (2 * self._cus) // -(-T // 16), key_tiles // 4))
+            n_split = max(1, min(8 if tiles else 16, (2 * self._cus) // -(-T // tile_rows), key_tiles // 4))
             part_o = part_ml = None
             if n_split > 1:
                 part_o = torch.empty((T, n_split, H * dv), dtype=torch.float32, device=q.device)
@@ -775,7 +779,7 @@ class HipOps:
                 _ptr(q), _ptr(kpool), _ptr(vpool), _ptr(talk), _ptr(block_table), _c_int(block_table.shape[1]), _ptr(seq_q_start),
                 _ptr(seq_q_len), _ptr(seq_pos0), _c_int(S), _ptr(out), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv),
                 _c_int(page_size), _c_int(window or 0), _c_int(keep_first), _c_float(scale), _c_int(n_split), _ptr(part_o), _ptr(part_ml),
-                self._stream()))
+                _c_int(tile_rows), self._stream()))
             return out
         if self._plan("ms_talking_split_takes", H, KV, d, dv, page_size, lib=lib):
             # blocks that share a row's keys, as many as fill the chip: how many follows from the step's rows and the

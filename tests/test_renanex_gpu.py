@@ -242,7 +242,8 @@ def _attention_case(dtype, H, KV, d, dv, ps, lens_before, lens_now, window, keep
         q, _ = ops.talking_prepare(dev(rows).unsqueeze(0), dev(qn) if normed else None, dev(kn) if normed else None, 1e-5, dev(positions.int()), dev(inv) if rot else None, rot, factor,
                                    None, None, False, dev(slot_map.int()), kpool, vpool, H, KV, d, dv, ps)
         out = ops.talking_attention(q, kpool, vpool, dev(T_) if talk else None, dev(table[live]), i32(q_start), i32([start[s] for s in live]),
-                                    H, KV, d, dv, ps, window, keep, scale, i32([lens[s] for s in live]), tiles)
+                                    H, KV, d, dv, ps, window, keep, scale, None if tiles == "vector" else i32([lens[s] for s in live]),
+                                    tiles is True)
         if phase == "now":
             for i, s in enumerate(live):
                 got[s] = out[q_start[i]:q_start[i] + lens[s]].float().cpu()
@@ -273,11 +274,12 @@ def _attention_case(dtype, H, KV, d, dv, ps, lens_before, lens_now, window, keep
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("tiles", [False, True])
+@pytest.mark.parametrize("tiles", [False, True, "vector"])
 @pytest.mark.parametrize("H,KV,d,dv,rot", [(4, 2, 32, 16, 16), (6, 1, 24, 40, 24), (3, 3, 8, 8, 0), (8, 8, 64, 64, 32), (5, 1, 20, 12, 4),
                                            (12, 4, 48, 80, 48), (24, 3, 16, 128, 8), (32, 32, 40, 16, 40)])
 def test_talking_attention_kernels(dtype, H, KV, d, dv, rot, tiles):
-    """One row a block, and 16 rows a block on the matrix cores (sizes that kernel does not take run in the other)."""
+    """On the matrix cores one row a block and 16 rows a block, and on the vector units (sizes that the kernel on the
+    matrix cores does not take run there in every case)."""
     # prompts, portions of prompts that go on, and single decoded rows side by side; a window that crosses pages
     _attention_case(dtype, H, KV, d, dv, 16, [0, 40, 70, 5], [50, 13, 1, 1], 24, 3, rot, True, seed=H, tiles=tiles)
     _attention_case(dtype, H, KV, d, dv, 16, [0, 31], [130, 1], None, 0, rot, H % 2 == 0, seed=H + 1, tiles=tiles)    # all keys, far ones too
@@ -287,7 +289,7 @@ def test_talking_attention_kernels(dtype, H, KV, d, dv, rot, tiles):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("decoded", [False, True, "tiles"])
+@pytest.mark.parametrize("decoded", [False, True, "tiles", "vector"])
 @pytest.mark.parametrize("edge", ["inside the window", "outside the window", "kept", "not kept", "page border", "own"])
 def test_a_key_that_stands_out_shows_at_every_edge(dtype, decoded, edge):
     """One key's score is made huge: its value is the output if the row sees it, and absent if not, so a window or
@@ -295,9 +297,9 @@ def test_a_key_that_stands_out_shows_at_every_edge(dtype, decoded, edge):
     window, keep, ps, n = 20, 5, 16, 64
     key = {"inside the window": n - window, "outside the window": n - window - 1, "kept": keep - 1, "not kept": keep,
            "page border": 48, "own": n - 1}[edge]
-    before, now = ([n - 1], [1]) if decoded is True else ([0], [n])
+    before, now = ([n - 1], [1]) if decoded in (True, "vector") else ([0], [n])
     got = _attention_case(dtype, 4, 2, 16, 16, ps, before, now, window, keep, 0, True, seed=11, spike=(0, key), normed=False,
-                          tiles=decoded == "tiles")
+                          tiles=True if decoded == "tiles" else "vector" if decoded == "vector" else False)
     assert len(got) == 1
 
 
