@@ -150,21 +150,31 @@ __global__ __launch_bounds__(256) void norm_add_kernel(float* __restrict__ x, co
     extern __shared__ float vals[];  // d floats: the summed row
     const size_t r = blockIdx.x;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < d; c += 256) {
-        // eight sums are asked for at once and added in order: one trip to memory for eight, not eight trips
-        const float* src = partials + r * d + c;
-        float v = 0.f;
-        int p = 0;
-        for (; p + 8 <= n_partials; p += 8) {
-            float q[8];
+    if (d % 4 == 0 && partial_stride % 4 == 0) {
+        // four columns a thread and up to eight sums asked for at once, added in order: few trips to memory a row
+        for (int c = threadIdx.x * 4; c < d; c += 1024) {
+            const float* src = partials + r * d + c;
+            f32x4 v = (f32x4){0.f, 0.f, 0.f, 0.f};
+            int p = 0;
+            for (; p + 8 <= n_partials; p += 8) {
+                f32x4 q[8];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) q[k] = src[(size_t)(p + k) * partial_stride];
+                for (int k = 0; k < 8; ++k) q[k] = *reinterpret_cast<const f32x4*>(src + (size_t)(p + k) * partial_stride);
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v += q[k];
+                for (int k = 0; k < 8; ++k) v += q[k];
+            }
+            for (; p < n_partials; ++p) v += *reinterpret_cast<const f32x4*>(src + (size_t)p * partial_stride);
+            *reinterpret_cast<f32x4*>(vals + c) = v;
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
         }
-        for (; p < n_partials; ++p) v += src[(size_t)p * partial_stride];
-        vals[c] = v;
-        ss += v * v;
+    } else {
+        for (int c = threadIdx.x; c < d; c += 256) {
+            const float* src = partials + r * d + c;
+            float v = 0.f;
+            for (int p = 0; p < n_partials; ++p) v += src[(size_t)p * partial_stride];
+            vals[c] = v;
+            ss += v * v;
+        }
     }
     ss = block_sum<256>(ss, scratch);
     const float inv = 1.0f / sqrtf(ss / (float)d + eps);

@@ -46,12 +46,13 @@ def close(got, want, dtype, what="", scale_by=None):
 def test_norm_add_and_softcap(dtype):
     ops = ops_of(dtype)
     torch.manual_seed(0)
-    x, parts, w = torch.randn(5, 72), torch.randn(3, 5, 72), torch.randn(72)
-    y = parts.double().sum(0)
-    want = x.double() + P.rms(y, 1e-5) * w.double()
-    xd = dev(x)
-    ops.norm_add(xd, dev(parts), dev(w), 1e-5)
-    close(xd, want, torch.float32, "norm_add")
+    for rows, width, sums in ((5, 72, 3), (3, 70, 1), (17, 2048, 19)):   # four columns a thread, or one where the width is odd
+        x, parts, w = torch.randn(rows, width), torch.randn(sums, rows, width), torch.randn(width)
+        y = parts.double().sum(0)
+        want = x.double() + P.rms(y, 1e-5) * w.double()
+        xd = dev(x)
+        ops.norm_add(xd, dev(parts), dev(w), 1e-5)
+        close(xd, want, torch.float32, f"norm_add of {sums} sums of width {width}")
     logits = torch.randn(4, 333) * 20
     ld = dev(logits)
     ops.softcap(ld, 0.25, 7.0)
