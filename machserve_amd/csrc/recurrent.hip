@@ -4,10 +4,13 @@
 //
 // A step's rows are the tokens of several requests, each request's rows contiguous and in order
 // (seq_q_start, seq_q_len); a request's state lives in slot seq_slot[s] of an array [slots, ...] of 32-bit
-// floats and is read at the start of the request's rows and written back after its last row.  Every request
-// is walked token after token in one fixed order, so what a token gets does not depend on how the tokens were
-// cut into steps or on what else the step holds.  Decays, step sizes, exponentials and the states themselves
-// are 32-bit in every build; the element type only stores the projections' outputs.
+// floats and is read at the start of the request's rows and written back after its last row.  A decoded token
+// is one step of the recurrence; a long portion is cut into pieces that are walked side by side (each from
+// zero, then the states between the pieces, then each from its own), and lightning attention takes 32 tokens
+// at a time on the matrix cores: the same sums in another order, so what a token gets depends on how the
+// tokens were cut into steps by rounding only, and never on what else the step holds.  Decays, step sizes,
+// exponentials, the states and all sums are 32-bit in every build; the element type stores the projections'
+// outputs and is the operand type of lightning attention's products.
 #include "common.cuh"
 
 namespace ms {

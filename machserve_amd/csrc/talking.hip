@@ -1,12 +1,17 @@
 // Attention whose heads exchange scores before the softmax ("talking heads"), over the paged cache, for a
 // window that keeps a request's first tokens, keys and values of different widths, a norm over the whole
 // query and key projections, a rotation of the first part of a head, and values blended with another
-// layer's.  Two kernels: one finishes a row of the q/k/v product (norm, rotation, blend) and writes its key
-// and value into their pages; the other is the attention of one row over the keys it sees.
+// layer's.  One kernel finishes a row of the q/k/v product (norm, rotation, blend) and writes its key and
+// value into their pages.  The attention itself runs on the matrix cores, 16 rows and every head a block for
+// steps of many rows and one row a block for decoding, several blocks sharing a tile's keys where tiles are
+// few (a last kernel merges their shares); and on the vector units, one row a block, for the head sizes and
+// counts that kernel does not take.
 //
-// Scores, the exchange between heads, the softmax and the weighted sum of values are 32-bit in every build;
-// so are the norm's statistics, angles, cosines and sines.  A row's result depends on its own keys alone
-// and is summed in one fixed order: it does not depend on what else the step holds.
+// Scores, the exchange between heads, the softmax and every sum are 32-bit in every build; so are the norm's
+// statistics, angles, cosines and sines.  The softmax weights are rounded to the element type only as an
+// operand of the product with the values on the matrix cores (not in the 32-bit build, and not on the vector
+// units).  A row's result depends on its own keys alone; which kernel runs, and how many blocks share a
+// row's keys, follows from the step's shape, and the kernels differ in rounding only.
 #include "common.cuh"
 
 namespace ms {
