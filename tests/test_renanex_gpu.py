@@ -458,13 +458,12 @@ def test_command_line_generates_from_a_folder_and_from_a_configuration(tmp_path)
     d = U.make_dir(tmp_path, "stateful", seed=15)
     w, cfg = U.read(d)
     prompt = U.tokens_of(9, 61, 4)
-    cmd = [sys.executable, os.path.join(root, "bin", "machserve"), "--prompt-ids", ",".join(map(str, prompt)), "--max-new", "5", "--dtype", "f32",
-           "--tpp", "16"]
-    r = subprocess.run(cmd + ["--model", d], capture_output=True, text=True, timeout=600)
+    cmd = [sys.executable, os.path.join(root, "bin", "machserve"), "--max-new", "5", "--dtype", "f32", "--tpp", "16", "--prompt-ids"]
+    r = subprocess.run(cmd + [",".join(map(str, prompt)), "--model", d], capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
     assert [int(t) for t in r.stdout.split()] == P.greedy_generate(w, cfg, prompt, 5, torch.float64)
     path = tmp_path / "config.json"
     path.write_text(json.dumps(U.CONFIGS["narrow"]))
-    r = subprocess.run(cmd + ["--random-config", str(path), "--weights-seed", "3"], capture_output=True, text=True, timeout=600)
+    r = subprocess.run(cmd + ["7,49,0,12", "--random-config", str(path), "--weights-seed", "3"], capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-2000:]
     assert len(r.stdout.split()) == 5 and all(0 <= int(t) < 50 for t in r.stdout.split())
