@@ -56,6 +56,9 @@ class RotarySpec:
     rotary_dim: Optional[int] = None
     # the precision in which the table of frequencies is worked out before it is rounded to 32-bit
     table_precision: str = "float32"
+    # which numbers of the rotated part make a pair: "halves" (j, j + rotary_dim/2) or "neighbours" (2j, 2j + 1); the
+    # table of frequencies is the same, the pairing is the business of the mixer's kernel
+    pairing: str = "halves"
 
 
 @dataclass(frozen=True)
@@ -105,6 +108,55 @@ class TalkingAttentionSpec:
     norm_eps: float = 1e-6
     talk: bool = True
     value_blend: Optional[str] = None
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class ConvAttentionSpec:
+    """Grouped-query attention whose values are its keys, behind a short convolution.
+
+    ``q = W_q h``, ``k = W_k h``; with ``conv_taps`` > 1 a causal convolution over time on every channel of q and k
+    (``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, no bias), whose last ``conv_taps - 1`` inputs are a request's state; the
+    values are the keys as they leave the convolution; with ``unit_norm`` q and k of every head are divided by their
+    root mean square (``norm_eps``, no weight); ``q_temp`` = (coef, every): the query at position p is multiplied by
+    ``1 + coef ln(floor((p + 1) / every) + 1)`` (None: not); ``score = scale q . k``, causal softmax; with ``gate`` head
+    h's output is multiplied by ``sigmoid(W_g h)_h``; output projection."""
+    kind: str
+    hidden: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    scale: float
+    conv_taps: int = 0
+    unit_norm: bool = True
+    norm_eps: float = 1e-6
+    q_temp: Optional[tuple] = None
+    gate: bool = True
+    tensors: Mapping[str, str] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention through a latent: per token the cache keeps an RMS-normed vector ``c`` of ``kv_rank`` numbers and one
+    rotated key part of ``rot_dim`` numbers that all heads share.  Queries come through a normed bottleneck of
+    ``q_rank``; a head's query is ``[head_dim plain | rot_dim rotated]``, its key ``[W_uk c | rotated part]``, its value
+    ``W_uv c`` (``v_head_dim``).  ``position`` describes the rotation of the ``rot_dim`` part (None: none); its cosines and
+    sines carry YaRN's factor, the plain part and ``scale`` do not.  ``sink``: the softmax's denominator also holds
+    ``exp(sink_h)``, a learned number per head without key or value.  ``kv_source``: index of another such layer whose
+    cache this layer reads (with its own ``W_uk``, ``W_uv``) instead of writing one."""
+    kind: str
+    hidden: int
+    heads: int
+    head_dim: int
+    rot_dim: int
+    v_head_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    position: Optional[RotarySpec]
+    norm_eps: float = 1e-6
+    sink: bool = False
+    kv_source: Optional[int] = None
     tensors: Mapping[str, str] = field(default_factory=dict)
 
 
@@ -169,6 +221,16 @@ class SandwichLayerSpec:
     mixer_post_norm: object
     feed_forward_norm: Optional[object]
     feed_forward_post_norm: Optional[object]
+
+
+@dataclass(frozen=True)
+class ParallelLayerSpec:
+    """A block whose branches read one norm: ``h = norm(x); x += mixer(h) + feed_forward(h)``; ``feed_forward`` None:
+    the layer has none."""
+    block: str
+    mixer: object
+    feed_forward: Optional[object]
+    norm: object
 
 
 @dataclass(frozen=True)

@@ -84,6 +84,11 @@ struct AttnArgs {
     int nsplit;
     float* part_o;   // [T, H, nsplit, hd]
     float* part_ml;  // [T, H, nsplit, 2]
+    // [H] or null: a softmax sink per head, a term exp(sink) in the denominator that has no key and no value
+    // (natural-logarithm units of the scaled scores)
+    const float* sinks;
+    // [T, H] or null: what the output of (row, head) is multiplied by (a gate), in the same pass as the softmax's division
+    const float* out_gate;
 };
 
 __device__ __forceinline__ float exp_f(float x) {
@@ -100,6 +105,18 @@ __device__ __forceinline__ float exp2_f(float x) {
 #else
     return exp2f(x);
 #endif
+}
+
+// What a row's unnormalised output is multiplied by at the end: 1 / l, or with a sink 1 / (l + exp(sink - m)), for a
+// running sum l taken relative to the maximum m (scaled scores, natural logarithm); a row without keys gives 0.
+// `gate`, if given, is the factor of this (row, head) on top of that.
+__device__ __forceinline__ float softmax_norm(float m, float l, const float* __restrict__ sinks, int head,
+                                              const float* __restrict__ gate, size_t row_head) {
+    const float g = gate ? gate[row_head] : 1.0f;
+    if (sinks == nullptr) return l > 0.f ? g / l : 0.f;
+    const float sk = sinks[head], top = fmaxf(m, sk);
+    const float c = l > 0.f ? exp_f(m - top) : 0.f;
+    return g * c / (l * c + exp_f(sk - top));
 }
 
 // KG "key groups" of four waves each share a block: group kg takes the key tiles whose absolute
@@ -489,7 +506,7 @@ __global__ __launch_bounds__(256 * KG, attention_waves_per_simd<KG>()) void page
     if (valid && a.nsplit > 1) {
         write_partial(acc_o, m_run, l_run);
     } else if (valid) {
-        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        const float inv = softmax_norm(m_run * a.scale, l_run, a.sinks, head, a.out_gate, (size_t)(q_start + tok) * a.H + head);
         elem_t* orow = a.out + ((size_t)(q_start + tok) * a.H + head) * hd;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) {
@@ -844,7 +861,7 @@ __global__ __launch_bounds__(r32::KG * r32::GT, 4) void paged_attention_rows32_k
     if (valid && a.nsplit > 1) {
         write_partial(acc, m_ref, l_run);
     } else if (valid) {
-        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        const float inv = softmax_norm(m_ref * a.scale, l_run, a.sinks, head, a.out_gate, (size_t)(q_start + tok) * a.H + head);
         elem_t* orow = a.out + ((size_t)(q_start + tok) * a.H + head) * hd;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt)
@@ -887,6 +904,8 @@ struct DecodeArgs {
     const float* inv_freq;   // [hd / 2] or null: no rotation
     const int* slot_map;     // [S] page * ps + offset of the row's key
     int n_partials, stride;
+    const float* sinks;      // [H] or null: see AttnArgs
+    const float* out_gate;   // [S, H] or null: see AttnArgs
 };
 
 constexpr int MAX_SPLITS = 64;
@@ -1273,7 +1292,7 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
     }
     if (!valid) return;
     if (a.nsplit == 1) {
-        const float inv = l_all > 0.f ? 1.0f / l_all : 0.f;
+        const float inv = softmax_norm(m_all, l_all, a.sinks, head, a.out_gate, (size_t)s * a.H + head);
         elem_t* orow = a.out + ((size_t)s * a.H + head) * hd;
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) {
@@ -1303,8 +1322,10 @@ __global__ __launch_bounds__(256) void decode_attention_kernel(DecodeArgs a) {
 // asked for eight at a time, the first eight together with the (max, sum) pairs and before anything
 // is computed from those, so that the kernel waits for memory once.
 __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                                          elem_t* __restrict__ out, int hd, int nsplit) {
-    arguments_now(part_o, part_ml, out, hd, nsplit);
+                                                          elem_t* __restrict__ out, int hd, int nsplit,
+                                                          const float* __restrict__ sinks, int H,
+                                                          const float* __restrict__ out_gate) {
+    arguments_now(part_o, part_ml, out, hd, nsplit, sinks, H, out_gate);
     constexpr int BATCH = 8;
     const size_t row = blockIdx.x;  // (request, head)
     const int lane = threadIdx.x;
@@ -1325,7 +1346,7 @@ __global__ __launch_bounds__(64) void decode_merge_kernel(const float* __restric
     const float c = lane < nsplit ? exp_f(m_own - m) : 0.f;
     float l = 0.f;
     for (int sp = 0; sp < nsplit; ++sp) l += __shfl(l_own * c, sp, WAVE);  // in split order
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    const float inv = softmax_norm(m, l, sinks, sinks ? (int)(row % (size_t)H) : 0, out_gate, row);
     const float coef = c * inv;  // of split `lane`; zero beyond the last split
     for (int d = lane; d - lane < hd; d += 64) {
         float o = 0.f;
@@ -1412,11 +1433,13 @@ extern "C" int MS_CAT(ms_attention_splits_nd, MS_ATTN_ND)(int n_work, int KV, in
     return (int)std::max(1L, std::min(n, (long)MAX_SPLITS));
 }
 
-extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
+// `sinks`: null, or one number per head that the softmax's denominator also holds as exp(sink); `out_gate`: null, or
+// float [T, H] that the output of each (row, head) is multiplied by.
+extern "C" int MS_CAT(ms_paged_attention_ex_nd, MS_ATTN_ND)(
     const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
     const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
     int hd, int ps, int n_pages, int window, float scale, int max_key_groups, int T, int nsplit, float* part_o,
-    float* part_ml, hipStream_t stream) {
+    float* part_ml, const float* sinks, const float* out_gate, hipStream_t stream) {
     MS_REQUIRE(n_work > 0, "attention: no work");
     MS_REQUIRE(nsplit >= 1 && nsplit <= MAX_SPLITS && (nsplit == 1 || (part_o && part_ml && T > 0)),
                "attention: %d key splits (at most %d, with their workspaces)", nsplit, MAX_SPLITS);
@@ -1426,7 +1449,7 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     MS_REQUIRE(window >= 0, "attention: window %d", window);
     MS_REQUIRE((double)n_pages * KV * ps * hd < 68719476736.0, "attention: a pool of %d pages exceeds 2^36 elements", n_pages);
     AttnArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, block_table, seq_q_start,
-               seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale, n_work, 0, nsplit, part_o, part_ml};
+               seq_q_len, seq_pos0, work, table_stride, H, KV, hd, ps, window, scale, n_work, 0, nsplit, part_o, part_ml, sinks, out_gate};
     // key groups per block by the longest context the block tables allow (the lengths themselves
     // are on the device): short contexts have no chain worth cutting
     const long span = window > 0 ? (long)window + BKV : (long)table_stride * ps;
@@ -1464,7 +1487,7 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
             hipLaunchKernelGGL(paged_attention_rows32_kernel, grid32, dim3(r32::KG * r32::GT), 0, stream, a);
             int rc32 = check_launch("paged_attention (32-row tiles)");
             if (rc32 || nsplit == 1) return rc32;
-            hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)((size_t)T * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
+            hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)((size_t)T * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit, a.sinks, H, a.out_gate);
             return check_launch("attention_merge");
         }
     }
@@ -1482,8 +1505,18 @@ extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
     }
     int rc = check_launch("paged_attention");
     if (rc || nsplit == 1) return rc;
-    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)((size_t)T * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
+    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)((size_t)T * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit, a.sinks, H, a.out_gate);
     return check_launch("attention_merge");
+}
+
+extern "C" int MS_CAT(ms_paged_attention_nd, MS_ATTN_ND)(
+    const void* q, const void* kpool, const void* vpool, void* out, const int* block_table, int table_stride,
+    const int* seq_q_start, const int* seq_q_len, const int* seq_pos0, const int* work, int n_work, int H, int KV,
+    int hd, int ps, int n_pages, int window, float scale, int max_key_groups, int T, int nsplit, float* part_o,
+    float* part_ml, hipStream_t stream) {
+    return MS_CAT(ms_paged_attention_ex_nd, MS_ATTN_ND)(q, kpool, vpool, out, block_table, table_stride, seq_q_start, seq_q_len,
+                                                          seq_pos0, work, n_work, H, KV, hd, ps, n_pages, window, scale,
+                                                          max_key_groups, T, nsplit, part_o, part_ml, nullptr, nullptr, stream);
 }
 
 extern "C" int MS_CAT(ms_attention_rows_per_block_nd, MS_ATTN_ND)() { return ROWS_PER_BLOCK; }
@@ -1491,22 +1524,30 @@ extern "C" int MS_CAT(ms_attention_rows_per_block_nd, MS_ATTN_ND)() { return ROW
 // Attention of a step in which every request has exactly one row (row s = request s).
 // part_o [S, H, nsplit, hd] and part_ml [S, H, nsplit, 2] are float workspaces (unused when
 // nsplit == 1).  Needs H / KV <= 16.
-extern "C" int MS_CAT(ms_decode_attention_nd, MS_ATTN_ND)(
+extern "C" int MS_CAT(ms_decode_attention_ex_nd, MS_ATTN_ND)(
     const void* q, const void* kpool, const void* vpool, void* out, float* part_o, float* part_ml, const int* block_table,
     int table_stride, const int* seq_pos0, int S, int H, int KV, int hd, int ps, int window, int nsplit, float scale,
-    hipStream_t stream) {
+    const float* sinks, const float* out_gate, hipStream_t stream) {
     MS_REQUIRE(S > 0, "decode attention: no rows");
     MS_REQUIRE(hd % 16 == 0 && hd > 0 && hd <= HDT, "decode attention: head size %d does not fit this tile of %d", hd, HDT);
     MS_REQUIRE(KV > 0 && H % KV == 0 && H / KV <= 16, "decode attention: %d heads over %d key/value heads (at most 16 each)", H, KV);
     MS_REQUIRE(ps % 16 == 0 && ps > 0, "decode attention: page size %d must be a multiple of 16", ps);
     MS_REQUIRE(nsplit >= 1 && nsplit <= MAX_SPLITS && (nsplit == 1 || (part_o && part_ml)), "decode attention: %d splits (at most %d)", nsplit, MAX_SPLITS);
     DecodeArgs a{(const elem_t*)q, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, part_o, part_ml, block_table,
-                 seq_pos0, table_stride, H, KV, hd, ps, window, nsplit, scale, nullptr, nullptr, nullptr, nullptr, 0, 0};
+                 seq_pos0, table_stride, H, KV, hd, ps, window, nsplit, scale, nullptr, nullptr, nullptr, nullptr, 0, 0, sinks, out_gate};
     hipLaunchKernelGGL(decode_attention_kernel<false>, dim3((unsigned)S, (unsigned)KV, (unsigned)nsplit), dim3(256), 0, stream, a);
     int rc = check_launch("decode_attention");
     if (rc || nsplit == 1) return rc;
-    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)(S * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
+    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)(S * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit, a.sinks, H, a.out_gate);
     return check_launch("decode_merge");
+}
+
+extern "C" int MS_CAT(ms_decode_attention_nd, MS_ATTN_ND)(
+    const void* q, const void* kpool, const void* vpool, void* out, float* part_o, float* part_ml, const int* block_table,
+    int table_stride, const int* seq_pos0, int S, int H, int KV, int hd, int ps, int window, int nsplit, float scale,
+    hipStream_t stream) {
+    return MS_CAT(ms_decode_attention_ex_nd, MS_ATTN_ND)(q, kpool, vpool, out, part_o, part_ml, block_table, table_stride, seq_pos0,
+                                                           S, H, KV, hd, ps, window, nsplit, scale, nullptr, nullptr, stream);
 }
 
 // Scratch memory of ms_decode_attention_noalloc_nd*: the splits' partial outputs, then their (max, sum)
@@ -1593,11 +1634,11 @@ extern "C" int MS_CAT(ms_decode_attention_fused_nd, MS_ATTN_ND)(
     MS_REQUIRE(nsplit >= 1 && nsplit <= MAX_SPLITS && (nsplit == 1 || (part_o && part_ml)), "decode attention: %d splits (at most %d)", nsplit, MAX_SPLITS);
     MS_REQUIRE(slot_map && kpool && vpool, "decode attention: the fused form writes the cache");
     DecodeArgs a{nullptr, (const elem_t*)kpool, (const elem_t*)vpool, (elem_t*)out, part_o, part_ml, block_table, seq_pos0,
-                 table_stride, H, KV, hd, ps, window, nsplit, scale, qkv, bias, inv_freq, slot_map, n_partials, stride};
+                 table_stride, H, KV, hd, ps, window, nsplit, scale, qkv, bias, inv_freq, slot_map, n_partials, stride, nullptr, nullptr};
     hipLaunchKernelGGL(decode_attention_kernel<true>, dim3((unsigned)S, (unsigned)KV, (unsigned)nsplit), dim3(256), 0, stream, a);
     int rc = check_launch("decode_attention_fused");
     if (rc || nsplit == 1) return rc;
-    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)(S * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit);
+    hipLaunchKernelGGL(decode_merge_kernel, dim3((unsigned)(S * H)), dim3(64), 0, stream, part_o, part_ml, (elem_t*)out, hd, nsplit, a.sinks, H, a.out_gate);
     return check_launch("decode_merge");
 }
 

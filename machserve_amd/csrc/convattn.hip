@@ -1,0 +1,163 @@
+// What grouped-query attention with a short convolution behind its projections needs around the paged attention
+// kernels: one row kernel that finishes a row of the fused projection [q | k | gate] from its 32-bit partial sums,
+// and the kernel that brings the convolution's state up to date.
+//
+// Per row: a causal convolution over time on every channel of q and k (the inputs before the step's first row of the
+// request come from the request's state, the last taps - 1 projected rows; before the request's start they are
+// zero); the values are the convolved keys as they are; q and k of every head are divided by their root mean square
+// (no weight); q is multiplied by a temperature that grows with the position,
+// 1 + coef * ln(floor((p + 1) / every) + 1); the gate's columns go through a sigmoid and are left as 32-bit
+// factors, one per (row, head), that the attention kernel applies to its output.  Keys and values are written into
+// the row's page, filled with zeros up to the attention tile's head size (the pools start as zeros; q's filling is
+// written).  Everything here is 32-bit; the element type is what q and the pages store.
+#include "common.cuh"
+
+namespace ms {
+
+__device__ __forceinline__ int seq_of_row(int t, const int* __restrict__ seq_q_start, int S) {
+    int lo = 0, hi = S - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (seq_q_start[mid] <= t) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
+}
+
+struct ConvRowArgs {
+    const float* proj;      // [n_partials, T, stride]: q [H, d], k [KV, d], gate [H] (gate only if gate_out)
+    int n_partials;
+    size_t partial_stride;
+    int stride;
+    const float* conv_w;    // [(H + KV) * d, taps] or null: no convolution
+    int taps;
+    const float* state;     // [slots, taps - 1, (H + KV) * d], oldest first
+    const int* seq_q_start;
+    const int* seq_slot;
+    int S;
+    const int* positions;   // [T]
+    int unit_norm;          // q and k of a head divided by their root mean square
+    float eps;
+    float temp_coef;        // 0: no temperature
+    int temp_every;
+    int values_are_keys;    // the value pool receives the keys before their norm
+    const int* slot_map;    // [T]
+    elem_t* q_out;          // [T, H, dp]
+    elem_t* kpool;          // [pages, KV, ps, dp]
+    elem_t* vpool;          // [pages, KV, dp, ps]
+    float* gate_out;        // [T, H] or null
+    int H, KV, d, dp, ps;
+};
+
+__global__ __launch_bounds__(256) void conv_row_kernel(ConvRowArgs a) {
+    extern __shared__ float row[];  // (H + KV) * d floats: the convolved row
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nq = a.H * a.d, C = (a.H + a.KV) * a.d;
+    const int s = seq_of_row(t, a.seq_q_start, a.S);
+    const int j = t - a.seq_q_start[s];
+    const int keep = a.taps - 1;
+    const float* st = a.conv_w ? a.state + (size_t)a.seq_slot[s] * keep * C : nullptr;
+    auto projected = [&](int r, int c) {
+        float v = 0.f;
+        for (int p = 0; p < a.n_partials; ++p) v += a.proj[p * a.partial_stride + (size_t)r * a.stride + c];
+        return v;
+    };
+    for (int c = threadIdx.x; c < C; c += 256) {
+        float y;
+        if (a.conv_w) {
+            y = 0.f;
+            for (int k = 0; k < a.taps; ++k) {
+                const int back = keep - k, idx = j - back;
+                const float u = idx >= 0 ? projected(t - back, c) : st[(size_t)(keep + idx) * C + c];
+                y += a.conv_w[(size_t)c * a.taps + k] * u;
+            }
+        } else {
+            y = projected(t, c);
+        }
+        row[c] = y;
+    }
+    if (a.gate_out)
+        for (int h = threadIdx.x; h < a.H; h += 256) a.gate_out[(size_t)t * a.H + h] = 1.0f / (1.0f + expf(-projected(t, C + h)));
+    __syncthreads();
+    const int pos = a.positions[t];
+    float temp = 1.0f;
+    if (a.temp_coef != 0.f) temp = 1.0f + a.temp_coef * logf((float)((pos + 1) / a.temp_every) + 1.0f);
+    const int slot = a.slot_map[t];
+    const int page = slot >= 0 ? slot / a.ps : 0, off = slot >= 0 ? slot % a.ps : 0;
+    // a wave a head: q heads first, then k heads
+    for (int hh = wave; hh < a.H + a.KV; hh += 4) {
+        const float* head = row + hh * a.d;
+        float ss = 0.f;
+        for (int e = lane; e < a.d; e += 64) ss += head[e] * head[e];
+        ss = wave_sum(ss);
+        const float inv = a.unit_norm ? 1.0f / sqrtf(ss / (float)a.d + a.eps) : 1.0f;
+        if (hh < a.H) {
+            elem_t* dst = a.q_out + ((size_t)t * a.H + hh) * a.dp;
+            for (int e = lane; e < a.dp; e += 64) dst[e] = from_f32<elem_t>(e < a.d ? head[e] * inv * temp : 0.f);
+        } else if (slot >= 0) {
+            const int kh = hh - a.H;
+            elem_t* krow = a.kpool + (((size_t)page * a.KV + kh) * a.ps + off) * a.dp;
+            elem_t* vcol = a.vpool + ((size_t)page * a.KV + kh) * a.dp * a.ps + off;
+            for (int e = lane; e < a.d; e += 64) {
+                krow[e] = from_f32<elem_t>(head[e] * inv);
+                if (a.values_are_keys) vcol[(size_t)e * a.ps] = from_f32<elem_t>(head[e]);
+            }
+        }
+    }
+}
+
+// The state after the step: the last taps - 1 projected rows of each request, old ones where the step brought fewer.
+constexpr int CONV_MAX_TAPS = 16;
+__global__ __launch_bounds__(256) void conv_row_state_kernel(const float* __restrict__ proj, int n_partials, size_t partial_stride, int stride,
+                                                             float* __restrict__ state, const int* __restrict__ seq_q_start,
+                                                             const int* __restrict__ seq_q_len, const int* __restrict__ seq_slot, int C,
+                                                             int taps) {
+    const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int n = seq_q_len[s], q0 = seq_q_start[s], keep = taps - 1;
+    float* st = state + (size_t)seq_slot[s] * keep * C;
+    float v[CONV_MAX_TAPS];
+    for (int i = 0; i < keep; ++i) {
+        const int idx = n - keep + i;  // among the step's rows; negative: an older input
+        float u = 0.f;
+        if (idx >= 0) {
+            for (int p = 0; p < n_partials; ++p) u += proj[p * partial_stride + (size_t)(q0 + idx) * stride + c];
+        } else {
+            u = st[(size_t)(keep + idx) * C + c];
+        }
+        v[i] = u;
+    }
+    for (int i = 0; i < keep; ++i) st[(size_t)i * C + c] = v[i];
+}
+
+}  // namespace ms
+
+using namespace ms;
+
+constexpr int CONV_MAX_ROW = 15000;
+extern "C" int ms_conv_rows_max_row() { return CONV_MAX_ROW; }
+extern "C" int ms_conv_rows_max_taps() { return CONV_MAX_TAPS; }
+
+// proj float [n_partials, T, stride]; conv_w null or float [(H + KV) * d, taps]; state float [slots, taps - 1, (H + KV) * d],
+// read here and brought up to date by a second launch; gate_out null or float [T, H].
+extern "C" int ms_conv_rows(const float* proj, int n_partials, int stride, const float* conv_w, int taps, float* state,
+                            const int* seq_q_start, const int* seq_q_len, const int* seq_slot, int S, const int* positions,
+                            int unit_norm, float eps, float temp_coef, int temp_every, int values_are_keys, const int* slot_map,
+                            void* q_out, void* kpool, void* vpool, float* gate_out, int T, int H, int KV, int d, int dp, int ps,
+                            hipStream_t stream) {
+    MS_REQUIRE(T > 0 && S > 0 && n_partials >= 1, "conv rows: %d rows of %d requests, %d partial sums", T, S, n_partials);
+    const int C = (H + KV) * d;
+    MS_REQUIRE(H > 0 && KV > 0 && d > 0 && dp >= d, "conv rows: %d heads, %d key/value heads, head size %d in %d", H, KV, d, dp);
+    MS_REQUIRE(stride >= C + (gate_out ? H : 0) && C <= CONV_MAX_ROW, "conv rows: a row of %d numbers (stride %d, at most %d)", C, stride, CONV_MAX_ROW);
+    MS_REQUIRE(!conv_w || (taps >= 2 && taps <= CONV_MAX_TAPS && state), "conv rows: %d taps (2 to %d, with a state)", taps, CONV_MAX_TAPS);
+    MS_REQUIRE(temp_coef == 0.f || temp_every > 0, "conv rows: temperature every %d positions", temp_every);
+    ConvRowArgs a{proj, n_partials, (size_t)T * stride, stride, conv_w, conv_w ? taps : 1, state, seq_q_start, seq_slot, S, positions,
+                  unit_norm, eps, temp_coef, temp_every, values_are_keys, slot_map, (elem_t*)q_out, (elem_t*)kpool, (elem_t*)vpool,
+                  gate_out, H, KV, d, dp, ps};
+    hipLaunchKernelGGL(conv_row_kernel, dim3(T), dim3(256), (size_t)C * sizeof(float), stream, a);
+    int rc = check_launch("conv_rows");
+    if (rc || !conv_w) return rc;
+    hipLaunchKernelGGL(conv_row_state_kernel, dim3(S, ceil_div(C, 256)), dim3(256), 0, stream, proj, n_partials, (size_t)T * stride, stride,
+                       state, seq_q_start, seq_q_len, seq_slot, C, taps);
+    return check_launch("conv_rows_state");
+}

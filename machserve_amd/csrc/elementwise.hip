@@ -57,6 +57,39 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(float* __restrict__ x, con
     for (int c = threadIdx.x; c < d; c += 256) dst[c] = from_f32<OutT>(vals[c] * inv);
 }
 
+// Layer norm with the same handling of rows and pending sums: v as above,
+// out[i, :] = (v - mean(v)) * rsqrt(mean((v - mean(v))^2) + eps) * w + b (b may be null).  The variance is the mean of
+// the squared deviations, taken in a second pass over the row in LDS.
+template <typename OutT>
+__global__ __launch_bounds__(256) void layernorm_kernel(float* __restrict__ x, const float* __restrict__ partials,
+                                                        int n_partials, size_t partial_stride,
+                                                        const int* __restrict__ rows, const float* __restrict__ w,
+                                                        const float* __restrict__ b, OutT* __restrict__ out, int d, float eps) {
+    __shared__ float scratch[4];
+    extern __shared__ float vals[];  // d floats: the summed row
+    const int i = blockIdx.x;
+    const size_t r = rows ? rows[i] : i;
+    float* src = x + r * d;
+    float sum = 0.f;
+    for (int c = threadIdx.x; c < d; c += 256) {
+        float v = src[c];
+        for (int p = 0; p < n_partials; ++p) v += partials[p * partial_stride + r * d + c];
+        if (n_partials > 0 && !rows) src[c] = v;
+        vals[c] = v;
+        sum += v;
+    }
+    const float mean = block_sum<256>(sum, scratch) / (float)d;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < d; c += 256) {
+        const float dv = vals[c] - mean;
+        ss += dv * dv;
+    }
+    ss = block_sum<256>(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+    OutT* dst = out + (size_t)i * d;
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] = from_f32<OutT>((vals[c] - mean) * inv * w[c] + (b ? b[c] : 0.f));
+}
+
 // The same for widths that are a multiple of four and at most 1024 * G.  A thread owns G groups of
 // four consecutive columns (group t, t + 256, ...) and asks for all of the row it needs - stream,
 // weights and the NP pending sums - before it uses the first value, so the kernel pays one memory
@@ -418,6 +451,21 @@ extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T
         hipLaunchKernelGGL(rmsnorm_kernel<elem_t>, dim3(n), dim3(256), smem, stream, x, partials, n_partials, ps, rows, w,
                            (elem_t*)out, d, eps);
     return check_launch("rmsnorm");
+}
+
+extern "C" int ms_layernorm(float* x, const float* partials, int n_partials, int T, const int* rows, const float* w, const float* b,
+                            void* out, int out_f32, int n, int d, float eps, hipStream_t stream) {
+    MS_REQUIRE(n > 0 && d > 0, "layernorm: empty problem n=%d d=%d", n, d);
+    MS_REQUIRE(d <= MAX_ROW_FLOATS, "layernorm: width %d exceeds the row buffer of %d", d, MAX_ROW_FLOATS);
+    MS_REQUIRE(n_partials == 0 || partials, "layernorm: %d partial sums without a buffer", n_partials);
+    const size_t ps = (size_t)T * d, smem = (size_t)d * sizeof(float);
+    if (out_f32 || !kHalf)
+        hipLaunchKernelGGL(layernorm_kernel<float>, dim3(n), dim3(256), smem, stream, x, partials, n_partials, ps, rows, w, b,
+                           (float*)out, d, eps);
+    else
+        hipLaunchKernelGGL(layernorm_kernel<elem_t>, dim3(n), dim3(256), smem, stream, x, partials, n_partials, ps, rows, w, b,
+                           (elem_t*)out, d, eps);
+    return check_launch("layernorm");
 }
 
 extern "C" int ms_norm_add(float* x, const float* partials, int n_partials, const float* w, int T, int d, float eps, hipStream_t stream) {

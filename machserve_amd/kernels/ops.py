@@ -160,6 +160,28 @@ class HipOps:
                                                       _c_float(eps), self._stream()))
         return out
 
+    def layernorm(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float,
+                  rows: Optional[torch.Tensor] = None, out_f32: bool = False, partials: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``(v - mean(v)) / sqrt(mean((v - mean(v))^2) + eps) * weight + bias`` for the rows ``v`` of ``x + sum(partials)``
+        (of its ``rows`` if given); with ``partials [P, T, d]`` and no ``rows`` the sum is also written back into ``x``."""
+        T, d = x.shape
+        self._want(x, torch.float32, "layernorm input")
+        self._want(weight, torch.float32, "layernorm weight", d)
+        if bias is not None:
+            self._want(bias, torch.float32, "layernorm bias", d)
+        n, P = T, 0
+        if rows is not None:
+            self._want(rows, torch.int32, "layernorm rows")
+            n = rows.numel()
+        if partials is not None:
+            P = partials.shape[0]
+            self._want(partials, torch.float32, "layernorm partial sums", P, T, d)
+        out = torch.empty((n, d), dtype=torch.float32 if out_f32 else self.dtype, device=x.device)
+        self._check(self._core, self._core.ms_layernorm(_ptr(x), _ptr(partials), _c_int(P), _c_int(T), _ptr(rows), _ptr(weight),
+                                                        _ptr(bias), _ptr(out), _c_int(int(out_f32)), _c_int(n), _c_int(d),
+                                                        _c_float(eps), self._stream()))
+        return out
+
     def add_partials(self, x: torch.Tensor, partials: torch.Tensor) -> None:
         """``x += sum(partials)`` in order."""
         T, d = x.shape
@@ -413,9 +435,9 @@ class HipOps:
         nd = build.attention_tile_for(hd)
         if nd not in self._attn:
             lib = self._load(build.ensure_library("attention", self.elem, nd))
-            self._attn[nd] = (lib, getattr(lib, f"ms_paged_attention_nd{nd}"),
+            self._attn[nd] = (lib, getattr(lib, f"ms_paged_attention_ex_nd{nd}"),
                               getattr(lib, f"ms_attention_rows_per_block_nd{nd}")(),
-                              getattr(lib, f"ms_decode_attention_nd{nd}"), getattr(lib, f"ms_attention_key_tile_nd{nd}")(),
+                              getattr(lib, f"ms_decode_attention_ex_nd{nd}"), getattr(lib, f"ms_attention_key_tile_nd{nd}")(),
                               getattr(lib, f"ms_decode_attention_fused_nd{nd}"))
         return self._attn[nd]
 
@@ -425,8 +447,11 @@ class HipOps:
     def paged_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                         seq_q_start: torch.Tensor, seq_q_len: torch.Tensor, seq_pos0: torch.Tensor,
                         work: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
-                        scale: float, max_key_groups: int = 0, key_splits: int = 0) -> torch.Tensor:
-        """``max_key_groups`` asks for that many groups of waves sharing a block's keys (0: the kernel's
+                        scale: float, max_key_groups: int = 0, key_splits: int = 0, sinks: Optional[torch.Tensor] = None,
+                        out_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``sinks`` float32 ``[H]``: the softmax's denominator also holds ``exp(sinks[h])``, a term without key or value;
+        ``out_gate`` float32 ``[T, H]``: what the output of each (row, head) is multiplied by, in the kernel's last pass.
+        ``max_key_groups`` asks for that many groups of waves sharing a block's keys (0: the kernel's
         choice); ``key_splits`` for that many blocks sharing them (0: the library's choice by the number of blocks
         of rows, the step's rows and the width of the block tables), merged by a second kernel."""
         lib, fn = self._attention_lib(hd)[:2]
@@ -436,6 +461,7 @@ class HipOps:
         self._want(kpool, self.dtype, "key pool", pages, KV, page_size, hd)
         self._want(vpool, self.dtype, "value pool", pages, KV, hd, page_size)
         S = seq_q_start.numel()
+        self._want_softmax_extras(sinks, out_gate, T, H)
         self._want(block_table, torch.int32, "block table")
         if block_table.dim() != 2 or block_table.shape[0] != S:
             raise KernelError(f"attention: block table {tuple(block_table.shape)} for {S} requests")
@@ -455,8 +481,14 @@ class HipOps:
                             _ptr(seq_q_start), _ptr(seq_q_len), _ptr(seq_pos0), _ptr(work), _c_int(work.shape[0]),
                             _c_int(H), _c_int(KV), _c_int(hd), _c_int(page_size), _c_int(pages), _c_int(window or 0),
                             _c_float(scale), _c_int(max_key_groups), _c_int(T), _c_int(nsplit), _ptr(part_o), _ptr(part_ml),
-                            self._stream()))
+                            _ptr(sinks), _ptr(out_gate), self._stream()))
         return out
+
+    def _want_softmax_extras(self, sinks, out_gate, T: int, H: int) -> None:
+        if sinks is not None:
+            self._want(sinks, torch.float32, "attention sinks", H)
+        if out_gate is not None:
+            self._want(out_gate, torch.float32, "attention output gate", T, H)
 
     DECODE_MAX_GROUP = 16  # query heads per key/value head the decode kernel takes
 
@@ -512,13 +544,15 @@ class HipOps:
 
     def decode_attention(self, q: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                          seq_pos0: torch.Tensor, H: int, KV: int, hd: int, page_size: int, window: Optional[int],
-                         scale: float) -> torch.Tensor:
-        """Attention of a step in which request ``s`` has the single row ``s``.  The keys are cut
+                         scale: float, sinks: Optional[torch.Tensor] = None, out_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Attention of a step in which request ``s`` has the single row ``s`` (``sinks``, ``out_gate``: see
+        :meth:`paged_attention`).  The keys are cut
         into splits so that the grid fills the chip; how many follows from the number of
         requests and the width of the block table only."""
         lib, _, _, fn, key_tile = self._attention_lib(hd)[:5]
         S = q.shape[0]
         self._want(q, self.dtype, "attention q", S, H * hd)
+        self._want_softmax_extras(sinks, out_gate, S, H)
         pages = kpool.shape[0]
         self._want(kpool, self.dtype, "key pool", pages, KV, page_size, hd)
         self._want(vpool, self.dtype, "value pool", pages, KV, hd, page_size)
@@ -536,7 +570,8 @@ class HipOps:
             part_ml = torch.empty((S, H, nsplit, 2), dtype=torch.float32, device=q.device)
         self._check(lib, fn(_ptr(q), _ptr(kpool), _ptr(vpool), _ptr(out), _ptr(part_o), _ptr(part_ml), _ptr(block_table),
                             _c_int(block_table.shape[1]), _ptr(seq_pos0), _c_int(S), _c_int(H), _c_int(KV), _c_int(hd),
-                            _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), self._stream()))
+                            _c_int(page_size), _c_int(window or 0), _c_int(nsplit), _c_float(scale), _ptr(sinks), _ptr(out_gate),
+                            self._stream()))
         return out
 
     # ------------------------------------------------------------------ a branch's output, normalised, into the stream
@@ -801,6 +836,120 @@ class HipOps:
             _ptr(seq_pos0), _c_int(S), _ptr(out), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dv), _c_int(page_size),
             _c_int(window or 0), _c_int(keep_first), _c_float(scale), self._stream()))
         return out
+
+    # ------------------------------------------------------------------ attention through a latent
+    def latent_limits(self) -> dict:
+        return {"row": self._extra_lib("latent").ms_latent_max_row()}
+
+    def latent_rows(self, proj: torch.Tensor, q_norm: torch.Tensor, c_norm: Optional[torch.Tensor], eps: float, positions: torch.Tensor,
+                    inv_freq: Optional[torch.Tensor], cs_factor: float, slot_map: Optional[torch.Tensor], kpool: Optional[torch.Tensor],
+                    vpool: Optional[torch.Tensor], q_rank: int, rank: int, rot: int, page_size: int) -> torch.Tensor:
+        """Finishes the rows of the down projections given as float32 partial sums ``[P, T, stride]`` (query latent
+        ``[q_rank]``, then, if the layer writes a cache (``c_norm`` given), latent ``[rank]`` and key part ``[rot]``): RMS
+        norm with weight of the query latent, returned ``[T, q_rank]`` in the element type; RMS norm with weight of the
+        latent, written as columns ``0 .. rank`` of the row's key and as the row's value; the key part rotated in pairs
+        ``(2i, 2i + 1)`` by ``positions * inv_freq`` with cosines and sines times ``cs_factor``, written behind it."""
+        lib = self._extra_lib("latent")
+        if proj.dim() == 2:
+            proj = proj.unsqueeze(0)
+        P, T, stride = proj.shape
+        self._want(proj, torch.float32, "latent rows")
+        self._want(q_norm, torch.float32, "query latent norm weight", q_rank)
+        hd = 0
+        if c_norm is not None:
+            self._want(c_norm, torch.float32, "latent norm weight", rank)
+            self._want(positions, torch.int32, "latent positions", T)
+            if rot:
+                self._want(inv_freq, torch.float32, "latent inv_freq", rot // 2)
+            self._want(slot_map, torch.int32, "latent slot_map", T)
+            pages, _, _, hd = kpool.shape
+            self._want(kpool, self.dtype, "latent key pool", pages, 1, page_size, hd)
+            self._want(vpool, self.dtype, "latent value pool", pages, 1, hd, page_size)
+        cq = torch.empty((T, q_rank), dtype=self.dtype, device=proj.device)
+        self._check(lib, lib.ms_latent_rows(_ptr(proj), _c_int(P), _c_int(stride), _ptr(q_norm), _ptr(c_norm), _c_float(eps),
+                                            _ptr(positions), _ptr(inv_freq), _c_float(cs_factor), _ptr(slot_map), _ptr(cq),
+                                            _ptr(kpool), _ptr(vpool), _c_int(T), _c_int(q_rank), _c_int(rank), _c_int(rot), _c_int(hd),
+                                            _c_int(page_size), self._stream()))
+        return cq
+
+    def latent_query(self, q: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], cs_factor: float, H: int, d: int,
+                     rot: int, rank: int, hd: int):
+        """From the up-projected queries ``q`` float32 ``[T, H * (d + rot)]``: ``(plain [T, H, dp], att [T, H, hd])`` in the
+        element type, ``dp`` = ``d`` rounded up to 8.  ``plain`` holds the heads' first ``d`` numbers; ``att``, the queries
+        of the attention over the latent cache, has its columns ``rank .. rank + rot`` set to the rotated rest and zeros
+        behind; its first ``rank`` columns are left for the per-head product to fill."""
+        lib = self._extra_lib("latent")
+        T = q.shape[0]
+        self._want(q, torch.float32, "latent queries", T, H * (d + rot))
+        self._want(positions, torch.int32, "latent positions", T)
+        if rot:
+            self._want(inv_freq, torch.float32, "latent inv_freq", rot // 2)
+        dp = -(-d // 8) * 8
+        plain = torch.empty((T, H, dp), dtype=self.dtype, device=q.device)
+        att = torch.empty((T, H, hd), dtype=self.dtype, device=q.device)
+        self._check(lib, lib.ms_latent_query(_ptr(q), _ptr(positions), _ptr(inv_freq), _c_float(cs_factor), _ptr(plain), _ptr(att),
+                                             _c_int(T), _c_int(H), _c_int(d), _c_int(dp), _c_int(rot), _c_int(rank), _c_int(hd),
+                                             self._stream()))
+        return plain, att
+
+    def heads_linear(self, a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """A product per head: ``out[t, b, :N] = w[b] @ a[t, b, :]`` for ``a [T, B, K]`` and ``w [B, N, K]``.  ``out``
+        ``[T, B, >= N]`` receives the result in its first ``N`` columns of every head (None: a new ``[T, B, N]``)."""
+        lib = self._extra_lib("latent")
+        T, B, K = a.shape
+        self._want(a, self.dtype, "heads_linear input")
+        self._want(w, self.dtype, "heads_linear weight", B, w.shape[1], K)
+        N = w.shape[1]
+        if out is None:
+            out = torch.empty((T, B, N), dtype=self.dtype, device=a.device)
+        self._want(out, self.dtype, "heads_linear output", T, B, out.shape[2])
+        if out.shape[2] < N:
+            raise KernelError(f"heads_linear: output heads of {out.shape[2]} columns for {N}")
+        self._check(lib, lib.ms_heads_linear(_ptr(a), ctypes.c_long(B * K), ctypes.c_long(K), _ptr(w), _ptr(out),
+                                             ctypes.c_long(B * out.shape[2]), ctypes.c_long(out.shape[2]), _c_int(T), _c_int(B), _c_int(N),
+                                             _c_int(K), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ attention behind a short convolution
+    def conv_rows_limits(self) -> dict:
+        lib = self._extra_lib("convattn")
+        return {"row": lib.ms_conv_rows_max_row(), "taps": lib.ms_conv_rows_max_taps()}
+
+    def conv_rows(self, proj: torch.Tensor, conv_w: Optional[torch.Tensor], state: Optional[torch.Tensor], seq_q_start: torch.Tensor,
+                  seq_q_len: torch.Tensor, seq_slot: torch.Tensor, positions: torch.Tensor, unit_norm: bool, eps: float,
+                  temp_coef: float, temp_every: int, values_are_keys: bool, gated: bool, slot_map: torch.Tensor, kpool: torch.Tensor,
+                  vpool: torch.Tensor, H: int, KV: int, d: int, page_size: int):
+        """Finishes the rows of a projection given as float32 partial sums ``[P, T, stride]`` (q ``[H, d]``, k ``[KV, d]``,
+        then with ``gated`` one gate column per head): causal convolution per channel with ``conv_w [(H + KV) * d, taps]``
+        over the request's earlier rows (``state [slots, taps - 1, (H + KV) * d]``, brought up to date; None: no
+        convolution), unit norm per head, the queries' temperature ``1 + temp_coef ln(floor((p + 1) / temp_every) + 1)``,
+        keys (and with ``values_are_keys`` the keys before their norm as values) written to their pages.  Returns
+        ``(q [T, H * dp]`` in the element type with ``dp`` the pools' head size, ``sigmoid(gate)`` float32 ``[T, H]`` or None)``."""
+        lib = self._extra_lib("convattn")
+        if proj.dim() == 2:
+            proj = proj.unsqueeze(0)
+        P, T, stride = proj.shape
+        C = (H + KV) * d
+        self._want(proj, torch.float32, "conv rows")
+        taps = 1
+        if conv_w is not None:
+            taps = conv_w.shape[1]
+            self._want(conv_w, torch.float32, "convolution weight", C, taps)
+            self._want(state, torch.float32, "convolution state", state.shape[0], taps - 1, C)
+        S = self._seq_operands("conv rows", seq_q_start, seq_q_len, seq_slot)
+        self._want(positions, torch.int32, "conv rows positions", T)
+        self._want(slot_map, torch.int32, "conv rows slot_map", T)
+        pages, _, _, dp = kpool.shape
+        self._want(kpool, self.dtype, "key pool", pages, KV, page_size, dp)
+        self._want(vpool, self.dtype, "value pool", pages, KV, dp, page_size)
+        q = torch.empty((T, H * dp), dtype=self.dtype, device=proj.device)
+        gate = torch.empty((T, H), dtype=torch.float32, device=proj.device) if gated else None
+        self._check(lib, lib.ms_conv_rows(_ptr(proj), _c_int(P), _c_int(stride), _ptr(conv_w), _c_int(taps), _ptr(state), _ptr(seq_q_start),
+                                          _ptr(seq_q_len), _ptr(seq_slot), _c_int(S), _ptr(positions), _c_int(int(unit_norm)), _c_float(eps),
+                                          _c_float(temp_coef), _c_int(temp_every), _c_int(int(values_are_keys)), _ptr(slot_map), _ptr(q),
+                                          _ptr(kpool), _ptr(vpool), _ptr(gate), _c_int(T), _c_int(H), _c_int(KV), _c_int(d), _c_int(dp),
+                                          _c_int(page_size), self._stream()))
+        return q, gate
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits, temperature, top_k, top_p, state, any_greedy: bool = True):

@@ -178,6 +178,17 @@ def require_kernel_sizes(rt: "Runtime", what: str, reductions=(), head_dim: Opti
         check(what, reductions, head_dim, norm_width, rotated_row)
 
 
+def attention_head_size(rt: "Runtime", size: int, unit: int = 64) -> int:
+    """The head size under which the paged attention kernels hold heads of ``size`` numbers (the rest is zeros): the
+    next multiple of 16 whose kernel takes work items of ``unit`` flat rows, so that mixers with heads of different
+    sizes can share a step's work lists."""
+    hd = -(-size // 16) * 16
+    per_block = getattr(rt.ops, "attention_rows_per_block", None)
+    while per_block is not None and per_block(hd) != unit:
+        hd += 16
+    return hd
+
+
 class Part:
     takes_pending_norm = False  # True: forward's normalised input may be a PendingNorm
 

@@ -1,4 +1,5 @@
-"""Arrangements of parts in a block.  Sandwich: a norm before and one after each branch,
+"""Arrangements of parts in a block.  Parallel: one norm feeds both branches, ``x += mixer(norm(x)) + feed_forward(norm(x))``.
+Sandwich: a norm before and one after each branch,
 ``x += post(mixer(pre(x))); x += post(feed_forward(pre(x)))``.  Pre-norm (``crates/mach-model/src/batched.rs:3180-3200,
 4031, 4050, 4453``): ``x += mixer(norm(x)); x += feed_forward(norm(x))``."""
 from __future__ import annotations
@@ -34,6 +35,27 @@ class PreNormBlock(Block):
             if pending is not None:
                 return pending
         return norm.forward(stream)
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """One norm for both branches, ``h = norm(x); x += mixer(h) + feed_forward(h)``.  Reads ``mixer``, ``feed_forward``
+    (may be None) and ``norm`` of its layer's spec.  Both branches end in a product that adds into the 32-bit stream."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.mixer = MIXERS.build(spec.mixer, rt)
+        self.norm = NORMS.build(spec.norm, rt)
+        self.feed_forward = FEED_FORWARDS.build(spec.feed_forward, rt) if spec.feed_forward is not None else None
+
+    def parts(self):
+        return [self.norm, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else [])
+
+    def forward(self, stream, ctx):
+        h = self.norm.forward(stream)  # a tensor: two readers share it
+        self.mixer.forward(h, stream, ctx)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(h, stream, ctx)
 
 
 class _Branch:

@@ -56,6 +56,29 @@ class ScalarRMSNorm(RMSNorm):
         self.weight = tensors["weight"].reshape(1).expand(self.spec.width).contiguous()
 
 
+@register_norm("layernorm")
+class LayerNorm(Norm):
+    """``y = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * weight + bias`` with 32-bit statistics; the bias is
+    optional in the checkpoint.  Pending sums of the stream are added by the norm's own kernel."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        require_kernel_sizes(rt, "layernorm", norm_width=spec.width)
+
+    def tensor_decls(self):
+        return [TensorDecl("weight", (self.spec.width,), "vector"), TensorDecl("bias", (self.spec.width,), "vector", optional=True)]
+
+    def load(self, tensors):
+        self.weight, self.bias = tensors["weight"], tensors.get("bias")
+
+    def forward(self, stream, rows=None):
+        stream.launch_deferred()
+        h = stream.ops.layernorm(stream.x, self.weight, self.bias, self.spec.eps, rows, False, stream.pending)
+        if rows is None:
+            stream.pending = None  # the kernel wrote the sum back
+        return h
+
+
 class PendingRMSNorm(PendingNorm):
     """The RMS norm left to its reader's first product, folded into it where the kernels take the shape."""
 
