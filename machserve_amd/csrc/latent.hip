@@ -30,7 +30,8 @@ struct LatentRowArgs {
     const float* inv_freq;  // [rot / 2]
     float cs_factor;        // what cosines and sines are multiplied by
     const int* slot_map;    // [T] page * ps + offset
-    elem_t* cq_out;         // [T, q_rank]
+    elem_t* cq_out;         // [T, cq_ld], zeros behind q_rank
+    int cq_ld;
     elem_t* kpool;          // [pages, 1, ps, hd]
     elem_t* vpool;          // [pages, 1, hd, ps]
     int q_rank, rank, rot, hd, ps;
@@ -56,7 +57,8 @@ __global__ __launch_bounds__(256) void latent_row_kernel(LatentRowArgs a) {
     ssc = block_sum<256>(ssc, scratch);
     __syncthreads();
     const float inv_q = 1.0f / sqrtf(ssq / (float)a.q_rank + a.eps);
-    for (int c = threadIdx.x; c < a.q_rank; c += 256) a.cq_out[(size_t)t * a.q_rank + c] = from_f32<elem_t>(row[c] * inv_q * a.q_norm[c]);
+    for (int c = threadIdx.x; c < a.cq_ld; c += 256)
+        a.cq_out[(size_t)t * a.cq_ld + c] = from_f32<elem_t>(c < a.q_rank ? row[c] * inv_q * a.q_norm[c] : 0.f);
     if (!kv) return;
     const int slot = a.slot_map[t];
     if (slot < 0) return;
@@ -177,8 +179,8 @@ extern "C" int ms_latent_max_row() { return LATENT_MAX_ROW; }
 // layer's cache); then slot_map, kpool, vpool, inv_freq are not read.
 extern "C" int ms_latent_rows(const float* proj, int n_partials, int stride, const float* q_norm, const float* c_norm, float eps,
                               const int* positions, const float* inv_freq, float cs_factor, const int* slot_map, void* cq_out,
-                              void* kpool, void* vpool, int T, int q_rank, int rank, int rot, int hd, int ps, hipStream_t stream) {
-    MS_REQUIRE(T > 0 && n_partials >= 1 && q_rank > 0, "latent rows: %d rows, %d partial sums, query latent of %d", T, n_partials, q_rank);
+                              int cq_ld, void* kpool, void* vpool, int T, int q_rank, int rank, int rot, int hd, int ps, hipStream_t stream) {
+    MS_REQUIRE(T > 0 && n_partials >= 1 && q_rank > 0 && cq_ld >= q_rank, "latent rows: %d rows, %d partial sums, query latent of %d in %d", T, n_partials, q_rank, cq_ld);
     const int n = q_rank + (c_norm ? rank + rot : 0);
     MS_REQUIRE(stride >= n && n <= LATENT_MAX_ROW, "latent rows: a row of %d numbers (stride %d, at most %d)", n, stride, LATENT_MAX_ROW);
     if (c_norm) {
@@ -186,7 +188,7 @@ extern "C" int ms_latent_rows(const float* proj, int n_partials, int stride, con
         MS_REQUIRE(positions && slot_map && kpool && vpool && (rot == 0 || inv_freq), "latent rows: the layer writes the cache");
     }
     LatentRowArgs a{proj, n_partials, (size_t)T * stride, stride, q_norm, c_norm, eps, positions, inv_freq, cs_factor, slot_map,
-                    (elem_t*)cq_out, (elem_t*)kpool, (elem_t*)vpool, q_rank, rank, rot, hd, ps};
+                    (elem_t*)cq_out, cq_ld, (elem_t*)kpool, (elem_t*)vpool, q_rank, rank, rot, hd, ps};
     hipLaunchKernelGGL(latent_row_kernel, dim3(T), dim3(256), (size_t)n * sizeof(float), stream, a);
     return check_launch("latent_rows");
 }

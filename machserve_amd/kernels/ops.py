@@ -846,7 +846,7 @@ class HipOps:
                     vpool: Optional[torch.Tensor], q_rank: int, rank: int, rot: int, page_size: int) -> torch.Tensor:
         """Finishes the rows of the down projections given as float32 partial sums ``[P, T, stride]`` (query latent
         ``[q_rank]``, then, if the layer writes a cache (``c_norm`` given), latent ``[rank]`` and key part ``[rot]``): RMS
-        norm with weight of the query latent, returned ``[T, q_rank]`` in the element type; RMS norm with weight of the
+        norm with weight of the query latent, returned ``[T, q_rank up to a multiple of 8]`` in the element type (zeros behind); RMS norm with weight of the
         latent, written as columns ``0 .. rank`` of the row's key and as the row's value; the key part rotated in pairs
         ``(2i, 2i + 1)`` by ``positions * inv_freq`` with cosines and sines times ``cs_factor``, written behind it."""
         lib = self._extra_lib("latent")
@@ -865,10 +865,10 @@ class HipOps:
             pages, _, _, hd = kpool.shape
             self._want(kpool, self.dtype, "latent key pool", pages, 1, page_size, hd)
             self._want(vpool, self.dtype, "latent value pool", pages, 1, hd, page_size)
-        cq = torch.empty((T, q_rank), dtype=self.dtype, device=proj.device)
+        cq = torch.empty((T, -(-q_rank // 8) * 8), dtype=self.dtype, device=proj.device)
         self._check(lib, lib.ms_latent_rows(_ptr(proj), _c_int(P), _c_int(stride), _ptr(q_norm), _ptr(c_norm), _c_float(eps),
                                             _ptr(positions), _ptr(inv_freq), _c_float(cs_factor), _ptr(slot_map), _ptr(cq),
-                                            _ptr(kpool), _ptr(vpool), _c_int(T), _c_int(q_rank), _c_int(rank), _c_int(rot), _c_int(hd),
+                                            _c_int(cq.shape[1]), _ptr(kpool), _ptr(vpool), _c_int(T), _c_int(q_rank), _c_int(rank), _c_int(rot), _c_int(hd),
                                             _c_int(page_size), self._stream()))
         return cq
 

@@ -33,8 +33,9 @@ class LatentAttention(Mixer):
             raise ValueError("latent_attention: the kernels rotate neighbouring pairs")
         self.hd = attention_head_size(rt, s.kv_rank + s.rot_dim)  # of the pools and of the attention kernels
         self.rank8 = -(-s.kv_rank // 8) * 8
-        require_kernel_sizes(rt, "latent_attention", [("hidden size", s.hidden), ("query latent", s.q_rank),
-                                                      ("heads x value size", s.heads * s.v_head_dim)], self.hd)
+        # the value size as the output projection sums over it: filled up where heads x value size is no multiple of 8
+        self.vd = s.v_head_dim if (s.heads * s.v_head_dim) % 8 == 0 else -(-s.v_head_dim // 8) * 8
+        require_kernel_sizes(rt, "latent_attention", [("hidden size", s.hidden)], self.hd)
         limits = getattr(rt.ops, "latent_limits", None)
         if limits is not None and s.q_rank + s.kv_rank + s.rot_dim > limits()["row"]:
             raise ValueError(f"latent_attention: a row of {s.q_rank + s.kv_rank + s.rot_dim} numbers exceeds the kernels' {limits()['row']}")
@@ -61,13 +62,13 @@ class LatentAttention(Mixer):
         pad = torch.nn.functional.pad
         self.w_down = torch.cat([t["dq.weight"], t["dkv.weight"]], dim=0).contiguous() if self.writes_cache else t["dq.weight"]
         self.q_norm, self.c_norm = t["dq.norm"], t.get("dkv.norm")
-        self.w_uq = t["uq.weight"]
+        self.w_uq = pad(t["uq.weight"], (0, -s.q_rank % 8)).contiguous()  # the query latent comes filled up to a multiple of 8
         d8 = -(-s.head_dim // 8) * 8
         # W_uk^T per head, [heads, kv_rank, head_dim (up to a multiple of 8)]: carries a plain query into the latent's space
         self.w_ukT = pad(t["uk.weight"].view(s.heads, s.head_dim, s.kv_rank).transpose(1, 2), (0, d8 - s.head_dim)).contiguous()
         # W_uv per head over the attention's head size, [heads, v_head_dim, hd]: zeros beside the latent's columns
         self.w_uv = pad(t["uv.weight"].view(s.heads, s.v_head_dim, s.kv_rank), (0, self.hd - s.kv_rank)).contiguous()
-        self.w_o = t["o.weight"]
+        self.w_o = pad(t["o.weight"].view(s.hidden, s.heads, s.v_head_dim), (0, self.vd - s.v_head_dim)).reshape(s.hidden, -1).contiguous()
         self.sink = t.get("sink")
 
     def cache_request(self):
@@ -107,5 +108,6 @@ class LatentAttention(Mixer):
             o = ops.paged_attention(att.view(att.shape[0], -1), self.kpool, self.vpool, view.block_table, ctx.seq_q_start, ctx.seq_q_len,
                                     ctx.seq_pos0, ctx.attention_work[s.heads], s.heads, 1, self.hd, view.page_size, None, float(s.scale),
                                     sinks=self.sink, out_gate=None)
-        y = ops.heads_linear(o.view(o.shape[0], s.heads, self.hd), self.w_uv)
+        y = o.new_zeros((o.shape[0], s.heads, self.vd)) if self.vd != s.v_head_dim else None
+        y = ops.heads_linear(o.view(o.shape[0], s.heads, self.hd), self.w_uv, y)
         stream.add_linear(y.view(y.shape[0], -1), self.w_o)

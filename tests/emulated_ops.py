@@ -124,8 +124,19 @@ class EmulatedOps:
     def attention_rows_per_block(self, hd):
         return self.rows_per_block
 
+    def layernorm(self, x, weight, bias, eps, rows=None, out_f32=False, partials=None):
+        full = x if partials is None else x + partials.sum(0)
+        if partials is not None and rows is None:
+            x.copy_(full)
+        src = full if rows is None else full[rows.long()]
+        dev = src - src.mean(-1, keepdim=True)
+        y = dev / torch.sqrt((dev * dev).mean(-1, keepdim=True) + eps) * weight
+        if bias is not None:
+            y = y + bias
+        return y if out_f32 else self._r(y)
+
     def paged_attention(self, q, kpool, vpool, block_table, seq_q_start, seq_q_len, seq_pos0, work, H, KV, hd,
-                        page_size, window, scale):
+                        page_size, window, scale, max_key_groups=0, key_splits=0, sinks=None, out_gate=None):
         T = q.shape[0]
         g = H // KV
         out = torch.zeros(T, H * hd)
@@ -147,8 +158,12 @@ class EmulatedOps:
                     kk = kpool[pages, kvh, offs, :].float()
                     vv = vpool[pages, kvh, :, offs].float()
                     sc = (kk @ q[qs + tok, h * hd:(h + 1) * hd].float()) * scale
-                    p = torch.softmax(sc, 0)
-                    out[qs + tok, h * hd:(h + 1) * hd] = p @ vv
+                    if sinks is not None:  # a term of the denominator without key or value
+                        p = torch.softmax(torch.cat([sc, sinks[h].reshape(1).float()]), 0)[:-1]
+                    else:
+                        p = torch.softmax(sc, 0)
+                    o = p @ vv
+                    out[qs + tok, h * hd:(h + 1) * hd] = o if out_gate is None else o * out_gate[qs + tok, h]
                     done.add((qs + tok, h))
         assert len(done) == T * H, "the work list does not cover every row and head"
         return self._r(out)
@@ -158,12 +173,94 @@ class EmulatedOps:
         q = self.rope_kv_write(qkv, bias, seq_pos0, inv_freq, slot_map, kpool, vpool, H, KV, hd, page_size)
         return self.decode_attention(q, kpool, vpool, block_table, seq_pos0, H, KV, hd, page_size, window, scale)
 
-    def decode_attention(self, q, kpool, vpool, block_table, seq_pos0, H, KV, hd, page_size, window, scale):
+    def decode_attention(self, q, kpool, vpool, block_table, seq_pos0, H, KV, hd, page_size, window, scale, sinks=None, out_gate=None):
         S = q.shape[0]
         ar = torch.arange(S, dtype=torch.int32)
         work = torch.stack([ar, torch.zeros_like(ar)], 1)
         return self.paged_attention(q, kpool, vpool, block_table, ar, torch.ones_like(ar), seq_pos0, work, H, KV, hd,
-                                    page_size, window, scale)
+                                    page_size, window, scale, sinks=sinks, out_gate=out_gate)
+
+    # ------------------------------------------------------------------ attention through a latent
+    def latent_limits(self):
+        return {"row": 15000}
+
+    @staticmethod
+    def _rotate_neighbours(x, positions, inv_freq, factor):
+        """``x [T, ..., rot]``: pairs (2i, 2i + 1) rotated by ``positions * inv_freq[i]``, cosines and sines times ``factor``."""
+        ang = positions.float().reshape([-1] + [1] * (x.dim() - 1)) * inv_freq.float()
+        c, sn = torch.cos(ang) * factor, torch.sin(ang) * factor
+        u, v = x[..., 0::2], x[..., 1::2]
+        return torch.stack([u * c - v * sn, v * c + u * sn], -1).flatten(-2)
+
+    def latent_rows(self, proj, q_norm, c_norm, eps, positions, inv_freq, cs_factor, slot_map, kpool, vpool, q_rank, rank, rot,
+                    page_size):
+        row = proj.sum(0) if proj.dim() == 3 else proj
+        T = row.shape[0]
+        rms = lambda x: x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+        cq = torch.zeros(T, -(-q_rank // 8) * 8)
+        cq[:, :q_rank] = rms(row[:, :q_rank]) * q_norm
+        if c_norm is not None:
+            c = self._r(rms(row[:, q_rank:q_rank + rank]) * c_norm)
+            page, off = (slot_map // page_size).long(), (slot_map % page_size).long()
+            kpool[page, 0, off, :rank] = c
+            vpool[page, 0, :rank, off] = c
+            if rot:
+                kpool[page, 0, off, rank:rank + rot] = self._r(self._rotate_neighbours(row[:, q_rank + rank:q_rank + rank + rot], positions,
+                                                                                       inv_freq, cs_factor))
+        return self._r(cq)
+
+    def latent_query(self, q, positions, inv_freq, cs_factor, H, d, rot, rank, hd):
+        T = q.shape[0]
+        qh = q.view(T, H, d + rot)
+        plain = torch.zeros(T, H, -(-d // 8) * 8)
+        plain[..., :d] = qh[..., :d]
+        att = torch.full((T, H, hd), float("nan"))  # the first `rank` columns are the per-head product's to fill
+        att[..., rank:] = 0.0
+        if rot:
+            att[..., rank:rank + rot] = self._rotate_neighbours(qh[..., d:], positions, inv_freq, cs_factor)
+        return self._r(plain), self._r(att)
+
+    def heads_linear(self, a, w, out=None):
+        y = torch.einsum("tbk,bnk->tbn", a.float(), w.float())
+        if out is None:
+            return self._r(y).contiguous()
+        out[..., :y.shape[-1]] = self._r(y)
+        return out
+
+    # ------------------------------------------------------------------ attention behind a short convolution
+    def conv_rows_limits(self):
+        return {"row": 15000, "taps": 16}
+
+    def conv_rows(self, proj, conv_w, state, seq_q_start, seq_q_len, seq_slot, positions, unit_norm, eps, temp_coef, temp_every,
+                  values_are_keys, gated, slot_map, kpool, vpool, H, KV, d, page_size):
+        row = proj.sum(0) if proj.dim() == 3 else proj
+        T, C, dp = row.shape[0], (H + KV) * d, kpool.shape[3]
+        y = row[:, :C].clone()
+        if conv_w is not None:
+            taps = conv_w.shape[1]
+            for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
+                hist = torch.cat([state[slot], row[q0:q0 + n, :C]], 0)  # the taps - 1 projected rows before, then the step's
+                acc = torch.zeros(n, C)
+                for k in range(taps):
+                    acc += hist[k:k + n] * conv_w[:, k]
+                y[q0:q0 + n] = acc
+                state[slot] = hist[n:]
+        q, k = y[:, :H * d].view(T, H, d), y[:, H * d:].view(T, KV, d)
+        v = k
+        if unit_norm:
+            rms = lambda x: x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+            q, k = rms(q), rms(k)
+        if temp_coef:
+            q = q * (1.0 + temp_coef * torch.log(torch.div(positions.long() + 1, temp_every, rounding_mode="floor").float() + 1.0))[:, None, None]
+        page, off = (slot_map // page_size).long(), (slot_map % page_size).long()
+        for h in range(KV):
+            kpool[page, h, off, :d] = self._r(k[:, h])
+            if values_are_keys:
+                vpool[page, h, :d, off] = self._r(v[:, h])
+        qo = torch.zeros(T, H, dp)
+        qo[..., :d] = q
+        gate = torch.sigmoid(row[:, C:C + H]) if gated else None
+        return self._r(qo).view(T, H * dp), gate
 
     def sample(self, logits, temperature, top_k, top_p, state, any_greedy=True):
         from plain.qwen2_plain import sample as plain_sample
