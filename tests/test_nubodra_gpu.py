@@ -128,7 +128,7 @@ def test_rows_behind_the_convolution_in_one_step_and_in_many(dtype, H, KV, d, ta
     C = (H + KV) * d
     lens = [11, 1, 6]
     T = sum(lens)
-    proj = torch.randn(2, T, C + 8)
+    proj = torch.randn(2, T, C + -(-H // 8) * 8)
     conv_w = torch.randn(C, taps) * 0.5 if taps else None
     coef, every = temp or (0.0, 1)
 
