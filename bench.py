@@ -299,6 +299,27 @@ def design_configs(z):
     return renanex, qwen
 
 
+def nubodra_configs(z):
+    """(Nubodra configuration, Qwen2 configuration) of one size: latent attention, two attention layers behind a
+    convolution, and a latent attention that reads the first one's cache, beside Qwen2 layers that see every key.  The
+    latent is as wide as the paged attention kernels' largest head allows beside a rotated part of 64 (192 + 64), the
+    queries' bottleneck three quarters of the width."""
+    w, H, kv, hd = z["width"], z["heads"], z["kv"], z["hd"]
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    lat = {"heads": H, "dim": hd, "rot_dim": 64, "vdim": hd, "q_rank": 3 * w // 4, "kv_rank": 192, "scale": (hd + 64) ** -0.5,
+           "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    att = {"type": "attention", "mlp": mlp, "mixer": {"heads": H, "kv_heads": kv, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "conv": 4,
+                                                       "q_temp": {"coef": 0.1, "every": 1024}}}
+    layers = [{"type": "latent_attention", "mlp": mlp, "mixer": dict(lat)}, att, att,
+              {"type": "latent_attention", "mlp": mlp, "mixer": dict(lat, kv_from=0)}]
+    nubodra = {"architecture": "Nubodra", "vocab": DESIGN_VOCAB, "width": w, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+               "layers": [dict(l, mixer=dict(l["mixer"], **({"kv_from": l["mixer"]["kv_from"] + 4 * r} if "kv_from" in l["mixer"] else {})))
+                          for r in range(z["layers"] // 4) for l in layers]}
+    qwen = design_configs(z)[1]
+    qwen.update(use_sliding_window=False)
+    return nubodra, qwen
+
+
 def compare_designs(args) -> int:
     """Prefill (one prompt in one step) and decode (a batch of single tokens at a context, from the captured step)
     of both designs through the step function; random weights, synthetic tokens.  One JSON line."""
@@ -313,7 +334,8 @@ def compare_designs(args) -> int:
     for size in args.design_sizes.split(","):
         z = DESIGN_SIZES[size]
         out[size] = {"sizes": z}
-        for name, raw in zip(("renanex", "qwen2"), design_configs(z)):
+        design = args.design
+        for name, raw in zip((design, "qwen2"), nubodra_configs(z) if design == "nubodra" else design_configs(z)):
             cfg = config_from_dict(raw)
             tensors = random_tensor_dict(cfg, 0, dt, device="cuda:0")
             page = args.page_size
@@ -346,10 +368,10 @@ def compare_designs(args) -> int:
                                "decode_tok_s": round(z["batch"] / decode, 1), "decode_ms": round(decode * 1e3, 4)}
             del lm, tensors
             torch.cuda.empty_cache()
-        r, q = out[size]["renanex"], out[size]["qwen2"]
-        out[size]["renanex_over_qwen2"] = {"prefill": round(r["prefill_tok_s"] / q["prefill_tok_s"], 3),
+        r, q = out[size][design], out[size]["qwen2"]
+        out[size][f"{design}_over_qwen2"] = {"prefill": round(r["prefill_tok_s"] / q["prefill_tok_s"], 3),
                                            "decode": round(r["decode_tok_s"] / q["decode_tok_s"], 3)}
-    print(json.dumps({"metric": "renanex_beside_qwen2_tokens_per_s", "dtype": args.dtype, "data": "synthetic", "steps": args.steps,
+    print(json.dumps({"metric": f"{args.design}_beside_qwen2_tokens_per_s", "dtype": args.dtype, "data": "synthetic", "steps": args.steps,
                       "warmup": args.warmup, "sizes": out}))
     return 0
 
@@ -377,6 +399,9 @@ def main() -> int:
     ap.add_argument("--designs", action="store_true",
                     help="instead of the default run: prefill and decode throughput of Renanex layers (Mamba scan, attention whose heads "
                          "exchange scores over a window, lightning attention) beside Qwen2 layers of equal sizes, at a few sizes")
+    ap.add_argument("--design", default="renanex", choices=["renanex", "nubodra"],
+                    help="with --designs: which design stands beside Qwen2 (nubodra: latent attention and attention behind a convolution, "
+                         "beside Qwen2 layers that see every key)")
     ap.add_argument("--design-sizes", default="small,medium", help="with --designs: which of the sizes to run (small, medium, large)")
     ap.add_argument("--record-calls", default=None, help=argparse.SUPPRESS)  # file that receives one step's operations (the traced run)
     args = ap.parse_args()

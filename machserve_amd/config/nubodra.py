@@ -64,7 +64,7 @@ def _mixer_of(kind: str, m: dict, where: str):
         q_temp = None
         if qt is not None:
             q_temp = (_num(qt, "coef", where + "q_temp.", positive=False), _int(qt, "every", where + "q_temp."))
-        return ConvAttentionLayer(heads, kv, dim, _num(m, "scale", where), 0 if conv == 1 else conv, q_temp)
+        return ConvAttentionLayer(heads, kv, dim, _num(m, "scale", where), conv, q_temp)
     if kind == "latent_attention":
         rot_dim = _int(m, "rot_dim", where, 0)
         rot = None

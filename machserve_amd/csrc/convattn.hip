@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void conv_row_kernel(ConvRowArgs a) {
     const int s = seq_of_row(t, a.seq_q_start, a.S);
     const int j = t - a.seq_q_start[s];
     const int keep = a.taps - 1;
-    const float* st = a.conv_w ? a.state + (size_t)a.seq_slot[s] * keep * C : nullptr;
+    const float* st = keep > 0 ? a.state + (size_t)a.seq_slot[s] * keep * C : nullptr;
     auto projected = [&](int r, int c) {
         float v = 0.f;
         for (int p = 0; p < a.n_partials; ++p) v += a.proj[p * a.partial_stride + (size_t)r * a.stride + c];
@@ -149,14 +149,14 @@ extern "C" int ms_conv_rows(const float* proj, int n_partials, int stride, const
     const int C = (H + KV) * d;
     MS_REQUIRE(H > 0 && KV > 0 && d > 0 && dp >= d, "conv rows: %d heads, %d key/value heads, head size %d in %d", H, KV, d, dp);
     MS_REQUIRE(stride >= C + (gate_out ? H : 0) && C <= CONV_MAX_ROW, "conv rows: a row of %d numbers (stride %d, at most %d)", C, stride, CONV_MAX_ROW);
-    MS_REQUIRE(!conv_w || (taps >= 2 && taps <= CONV_MAX_TAPS && state), "conv rows: %d taps (2 to %d, with a state)", taps, CONV_MAX_TAPS);
+    MS_REQUIRE(!conv_w || (taps >= 1 && taps <= CONV_MAX_TAPS && (state || taps == 1)), "conv rows: %d taps (1 to %d, with a state from 2 on)", taps, CONV_MAX_TAPS);
     MS_REQUIRE(temp_coef == 0.f || temp_every > 0, "conv rows: temperature every %d positions", temp_every);
     ConvRowArgs a{proj, n_partials, (size_t)T * stride, stride, conv_w, conv_w ? taps : 1, state, seq_q_start, seq_slot, S, positions,
                   unit_norm, eps, temp_coef, temp_every, values_are_keys, slot_map, (elem_t*)q_out, (elem_t*)kpool, (elem_t*)vpool,
                   gate_out, H, KV, d, dp, ps};
     hipLaunchKernelGGL(conv_row_kernel, dim3(T), dim3(256), (size_t)C * sizeof(float), stream, a);
     int rc = check_launch("conv_rows");
-    if (rc || !conv_w) return rc;
+    if (rc || !conv_w || taps < 2) return rc;
     hipLaunchKernelGGL(conv_row_state_kernel, dim3(S, ceil_div(C, 256)), dim3(256), 0, stream, proj, n_partials, (size_t)T * stride, stride,
                        state, seq_q_start, seq_q_len, seq_slot, C, taps);
     return check_launch("conv_rows_state");

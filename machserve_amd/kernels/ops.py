@@ -935,7 +935,10 @@ class HipOps:
         if conv_w is not None:
             taps = conv_w.shape[1]
             self._want(conv_w, torch.float32, "convolution weight", C, taps)
-            self._want(state, torch.float32, "convolution state", state.shape[0], taps - 1, C)
+            if taps > 1:
+                self._want(state, torch.float32, "convolution state", state.shape[0], taps - 1, C)
+            else:
+                state = None
         S = self._seq_operands("conv rows", seq_q_start, seq_q_len, seq_slot)
         self._want(positions, torch.int32, "conv rows positions", T)
         self._want(slot_map, torch.int32, "conv rows slot_map", T)

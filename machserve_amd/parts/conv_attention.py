@@ -24,7 +24,7 @@ class ConvAttention(Mixer):
         if s.heads % s.kv_heads:
             raise ValueError(f"conv_attention: {s.heads} heads are not a multiple of {s.kv_heads} key/value heads")
         self.nq, self.nk = s.heads * s.head_dim, s.kv_heads * s.head_dim
-        self.taps = s.conv_taps if s.conv_taps and s.conv_taps > 1 else 0
+        self.taps = s.conv_taps or 0  # one tap is a weight per channel and needs no state
         self.hd = attention_head_size(rt, s.head_dim)  # of the pools and of the attention kernels
         require_kernel_sizes(rt, "conv_attention", [("hidden size", s.hidden)], self.hd)
         limits = getattr(rt.ops, "conv_rows_limits", None)
@@ -61,14 +61,14 @@ class ConvAttention(Mixer):
 
     def cache_request(self):
         pages = PagedKVRequest(self.spec.kv_heads, self.hd)
-        if not self.taps:
+        if self.taps < 2:
             return pages
         return [pages, StateRequest({"conv": (self.taps - 1, self.nq + self.nk)})]
 
     def bind_cache(self, binding):
-        pages = binding[0] if self.taps else binding
+        pages = binding[0] if self.taps > 1 else binding
         self.group, self.kpool, self.vpool = pages.group, pages.kpool, pages.vpool
-        self.state = binding[1].tensors["conv"] if self.taps else None
+        self.state = binding[1].tensors["conv"] if self.taps > 1 else None
 
     def attention_rows_per_token(self):
         return self.spec.heads // self.spec.kv_heads

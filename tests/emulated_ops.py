@@ -239,12 +239,14 @@ class EmulatedOps:
         if conv_w is not None:
             taps = conv_w.shape[1]
             for q0, n, slot in zip(seq_q_start.tolist(), seq_q_len.tolist(), seq_slot.tolist()):
-                hist = torch.cat([state[slot], row[q0:q0 + n, :C]], 0)  # the taps - 1 projected rows before, then the step's
+                before = state[slot] if taps > 1 else row.new_zeros(0, C)
+                hist = torch.cat([before, row[q0:q0 + n, :C]], 0)  # the taps - 1 projected rows before, then the step's
                 acc = torch.zeros(n, C)
                 for k in range(taps):
                     acc += hist[k:k + n] * conv_w[:, k]
                 y[q0:q0 + n] = acc
-                state[slot] = hist[n:]
+                if taps > 1:
+                    state[slot] = hist[n:]
         q, k = y[:, :H * d].view(T, H, d), y[:, H * d:].view(T, KV, d)
         v = k
         if unit_norm:

@@ -42,12 +42,12 @@ CONFIGS = {
         latent(2, 8, 8, 16, 16, 24, 0.5, scaling=YARN, kv_from=0, ff=72),
         conv_attention(3, 3, 16, 0.4, conv=2, q_temp=(0.2, 1), ff=None)]),
     # sizes that are no multiples of 8 or 16, one key/value head under six heads, five taps, two latent caches of
-    # different widths, a rotation without scaling, an attention without convolution or temperature
+    # different widths, a rotation without scaling, an attention with one tap (no state) and no temperature
     "odd": model(48, 61, [
         conv_attention(6, 1, 20, 0.3, conv=5, q_temp=(1.5, 7), ff=40),
         latent(3, 12, 6, 20, 20, 26, 0.4, base=500.0, ff=None),
         latent(5, 8, 4, 8, 12, 12, 0.6, base=100.0, scaling={"factor": 2.0, "original": 16, "fast": 4.0, "slow": 2.0}, ff=56),
-        conv_attention(2, 2, 8, 0.7, ff=24),
+        conv_attention(2, 2, 8, 0.7, conv=1, ff=24),
         latent(4, 4, 6, 6, 9, 26, 0.5, base=500.0, kv_from=1, ff=32)], eps=1e-6, scale=1.0),
     # more heads than a decode tile holds over one latent, more than a few heads a key/value head
     "heads": model(64, 80, [

@@ -119,7 +119,7 @@ def test_rotation_of_the_latent_kernels_is_the_plain_models():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,KV,d,taps,temp", [(4, 2, 24, 4, (0.7, 5)), (6, 1, 20, 5, (1.5, 7)), (3, 3, 16, 2, (0.2, 1)), (2, 2, 8, 0, None),
+@pytest.mark.parametrize("H,KV,d,taps,temp", [(4, 2, 24, 4, (0.7, 5)), (6, 1, 20, 5, (1.5, 7)), (3, 3, 16, 2, (0.2, 1)), (2, 2, 8, 0, None), (2, 2, 8, 1, None),
                                               (18, 1, 16, 3, (0.5, 16)), (2, 1, 72, 7, (0.3, 128))])
 def test_rows_behind_the_convolution_in_one_step_and_in_many(dtype, H, KV, d, taps, temp):
     ops, ref = ops_of(dtype), EmulatedOps(dtype)
@@ -134,7 +134,7 @@ def test_rows_behind_the_convolution_in_one_step_and_in_many(dtype, H, KV, d, ta
 
     def run(o, cuts, to):
         """The three requests' rows in steps of the given sizes (a request's share of a step: its next `cut` rows)."""
-        state = to(torch.zeros(5, max(taps - 1, 1), C))[:, :taps - 1].contiguous() if taps else None
+        state = to(torch.zeros(5, taps - 1, C)) if taps > 1 else None
         kp, vp = to(torch.zeros(6, KV, ps, hd, dtype=dtype)), to(torch.zeros(6, KV, hd, ps, dtype=dtype))
         qs, gates = [None] * T, [None] * T
         starts = [0, lens[0], lens[0] + lens[1]]
