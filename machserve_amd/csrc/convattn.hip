@@ -106,6 +106,115 @@ __global__ __launch_bounds__(256) void conv_row_kernel(ConvRowArgs a) {
     }
 }
 
+// The same with a wave a head and R consecutive rows of the step a block, for up to FAST_TAPS taps and heads of up to
+// 256 numbers: a lane holds its channels' projected rows t0 - (taps - 1) .. t0 + R - 1 in registers (each row of the
+// projection is read (R + taps - 1) / R times instead of `taps` times), all loads of a chunk are asked for before the
+// first is used, and a head's sum of squares is a reduction over the wave: no LDS and no barrier.  R = 8 in steps of
+// many rows, 1 where rows are few (decoding: the blocks would not fill the chip otherwise, and a row's earlier inputs
+// come from its request's state anyway).  The gate's columns are one more "head".  Same sums in the same order as the
+// kernel above.
+constexpr int FAST_TAPS = 8, FAST_CHUNKS = 4;
+template <int R>
+__global__ __launch_bounds__(256) void conv_head_kernel(ConvRowArgs a, int T) {
+    constexpr int W = R + FAST_TAPS - 1;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int hh = blockIdx.y * 4 + wave, t0 = blockIdx.x * R;
+    const int n_heads = a.H + a.KV;
+    if (hh > n_heads || (hh == n_heads && !a.gate_out)) return;  // the same for the whole wave; the kernel has no barrier
+    const int C = n_heads * a.d;
+    auto projected = [&](int r, int c) {
+        float v = 0.f;
+        for (int p = 0; p < a.n_partials; ++p) v += a.proj[p * a.partial_stride + (size_t)r * a.stride + c];
+        return v;
+    };
+    if (hh == n_heads) {
+        for (int i = 0; i < R; ++i) {
+            const int t = t0 + i;
+            if (t >= T) break;
+            for (int h = lane; h < a.H; h += 64) a.gate_out[(size_t)t * a.H + h] = 1.0f / (1.0f + expf(-projected(t, C + h)));
+        }
+        return;
+    }
+    const int keep = a.taps - 1;
+    // per row of the block: how many rows of its request the step holds before it, and the request's state
+    int before[R];
+    const float* st[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int t = min(t0 + i, T - 1);
+        const int s = seq_of_row(t, a.seq_q_start, a.S);
+        before[i] = t - a.seq_q_start[s];
+        st[i] = keep > 0 ? a.state + (size_t)a.seq_slot[s] * keep * C : nullptr;
+    }
+    float y[FAST_CHUNKS][R];
+#pragma unroll
+    for (int ci = 0; ci < FAST_CHUNKS; ++ci) {
+        const int e = lane + 64 * ci;
+        const bool live = e < a.d;  // the same for the wave's later chunks too: they are skipped whole
+        if (ci * 64 >= a.d) {
+#pragma unroll
+            for (int i = 0; i < R; ++i) y[ci][i] = 0.f;
+            continue;
+        }
+        const int c = hh * a.d + (live ? e : 0);
+        float win[W], cw[FAST_TAPS];
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+            const int r = t0 - keep + w;
+            win[w] = (w < R + keep && r >= 0 && r < T) ? projected(r, c) : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < FAST_TAPS; ++k) cw[k] = k < a.taps ? (a.conv_w ? a.conv_w[(size_t)c * a.taps + k] : 1.0f) : 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            float acc = 0.f;
+#pragma unroll
+            for (int k = 0; k < FAST_TAPS; ++k) {
+                if (k < a.taps) {
+                    // tap k reads the row (taps - 1 - k) back: of this step if the request has that many rows before, else of its state
+                    const float u = k >= keep - before[i] ? win[i + k] : st[i][(size_t)(before[i] + k) * C + c];
+                    acc += cw[k] * u;
+                }
+            }
+            y[ci][i] = live ? acc : 0.f;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int t = t0 + i;
+        if (t >= T) break;
+        float ss = 0.f;
+#pragma unroll
+        for (int ci = 0; ci < FAST_CHUNKS; ++ci) ss += y[ci][i] * y[ci][i];
+        ss = wave_sum(ss);
+        const float inv = a.unit_norm ? 1.0f / sqrtf(ss / (float)a.d + a.eps) : 1.0f;
+        if (hh < a.H) {
+            float temp = 1.0f;
+            if (a.temp_coef != 0.f) temp = 1.0f + a.temp_coef * logf((float)((a.positions[t] + 1) / a.temp_every) + 1.0f);
+            elem_t* dst = a.q_out + ((size_t)t * a.H + hh) * a.dp;
+#pragma unroll
+            for (int ci = 0; ci < FAST_CHUNKS; ++ci) {
+                const int e = lane + 64 * ci;
+                if (e < a.dp) dst[e] = from_f32<elem_t>(e < a.d ? y[ci][i] * inv * temp : 0.f);
+            }
+        } else {
+            const int slot = a.slot_map[t];
+            if (slot < 0) continue;
+            const int page = slot / a.ps, off = slot % a.ps, kh = hh - a.H;
+            elem_t* krow = a.kpool + (((size_t)page * a.KV + kh) * a.ps + off) * a.dp;
+            elem_t* vcol = a.vpool + ((size_t)page * a.KV + kh) * a.dp * a.ps + off;
+#pragma unroll
+            for (int ci = 0; ci < FAST_CHUNKS; ++ci) {
+                const int e = lane + 64 * ci;
+                if (e < a.d) {
+                    krow[e] = from_f32<elem_t>(y[ci][i] * inv);
+                    if (a.values_are_keys) vcol[(size_t)e * a.ps] = from_f32<elem_t>(y[ci][i]);
+                }
+            }
+        }
+    }
+}
+
 // The state after the step: the last taps - 1 projected rows of each request, old ones where the step brought fewer.
 constexpr int CONV_MAX_TAPS = 16;
 __global__ __launch_bounds__(256) void conv_row_state_kernel(const float* __restrict__ proj, int n_partials, size_t partial_stride, int stride,
@@ -154,7 +263,13 @@ extern "C" int ms_conv_rows(const float* proj, int n_partials, int stride, const
     ConvRowArgs a{proj, n_partials, (size_t)T * stride, stride, conv_w, conv_w ? taps : 1, state, seq_q_start, seq_slot, S, positions,
                   unit_norm, eps, temp_coef, temp_every, values_are_keys, slot_map, (elem_t*)q_out, (elem_t*)kpool, (elem_t*)vpool,
                   gate_out, H, KV, d, dp, ps};
-    hipLaunchKernelGGL(conv_row_kernel, dim3(T), dim3(256), (size_t)C * sizeof(float), stream, a);
+    if (a.taps <= FAST_TAPS && dp <= 64 * FAST_CHUNKS) {
+        const int units = ceil_div(H + KV + (gate_out ? 1 : 0), 4);
+        if (T > 64) hipLaunchKernelGGL(conv_head_kernel<8>, dim3(ceil_div(T, 8), units), dim3(256), 0, stream, a, T);
+        else hipLaunchKernelGGL(conv_head_kernel<1>, dim3(T, units), dim3(256), 0, stream, a, T);
+    } else {
+        hipLaunchKernelGGL(conv_row_kernel, dim3(T), dim3(256), (size_t)C * sizeof(float), stream, a);
+    }
     int rc = check_launch("conv_rows");
     if (rc || !conv_w || taps < 2) return rc;
     hipLaunchKernelGGL(conv_row_state_kernel, dim3(S, ceil_div(C, 256)), dim3(256), 0, stream, proj, n_partials, (size_t)T * stride, stride,

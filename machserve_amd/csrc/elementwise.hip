@@ -96,18 +96,20 @@ __global__ __launch_bounds__(256) void layernorm_kernel(float* __restrict__ x, c
 // round trip instead of one per column and pending sum.  The sums are added in the same order.
 // With more than eight pending sums (MORE, NP = 8) the rest, up to eight again, follows in a second
 // round of loads.
-template <typename OutT, int G, int NP, bool MORE = false>
+// With CENTER the row's mean is taken off before the squares are summed and `bias` (may be null) is added at the end:
+// a layer norm, (v - mean) * rsqrt(mean((v - mean)^2) + eps) * w + bias; the stream takes the sums as they are.
+template <typename OutT, int G, int NP, bool MORE = false, bool CENTER = false>
 __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x, const float* __restrict__ partials,
                                                            size_t partial_stride, const int* __restrict__ rows,
                                                            const float* __restrict__ w, OutT* __restrict__ out, int d,
-                                                           float eps, int n_more) {
-    arguments_now(x, partials, partial_stride, rows, w, out, d, eps, n_more);
+                                                           float eps, int n_more, const float* __restrict__ bias) {
+    arguments_now(x, partials, partial_stride, rows, w, out, d, eps, n_more, bias);
     __shared__ float scratch[4];
     const int i = blockIdx.x, ng = d / 4;
     const size_t r = rows ? rows[i] : i;
     f32x4* src = reinterpret_cast<f32x4*>(x + r * d);
     const f32x4* w4 = reinterpret_cast<const f32x4*>(w);
-    f32x4 v[G], wv[G], pend[NP > 0 ? NP : 1][G];
+    f32x4 v[G], wv[G], bv[G], pend[NP > 0 ? NP : 1][G];
     int at[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -115,6 +117,10 @@ __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x
         at[g] = c4 < ng ? c4 : 0;  // a group beyond the row reads group 0 and is dropped
         v[g] = src[at[g]];
         wv[g] = w4[at[g]];
+        bv[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if constexpr (CENTER) {
+            if (bias) bv[g] = reinterpret_cast<const f32x4*>(bias)[at[g]];
+        }
     }
 #pragma unroll
     for (int p = 0; p < NP; ++p)
@@ -140,7 +146,7 @@ __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x
                 v[g] += pend[p][g] * keep;
             }
     }
-    float ss = 0.f;
+    float ss = 0.f, sum = 0.f;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         if constexpr (!MORE) {
@@ -149,7 +155,16 @@ __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x
         }
         if (threadIdx.x + g * 256 < ng) {
             if ((NP > 0 || MORE) && !rows) src[at[g]] = v[g];
-            ss += v[g].x * v[g].x + v[g].y * v[g].y + v[g].z * v[g].z + v[g].w * v[g].w;
+            if constexpr (CENTER) sum += v[g].x + v[g].y + v[g].z + v[g].w;
+            else ss += v[g].x * v[g].x + v[g].y * v[g].y + v[g].z * v[g].z + v[g].w * v[g].w;
+        }
+    }
+    if constexpr (CENTER) {
+        const float mean = block_sum<256>(sum, scratch) / (float)d;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            v[g] -= mean;
+            if (threadIdx.x + g * 256 < ng) ss += v[g].x * v[g].x + v[g].y * v[g].y + v[g].z * v[g].z + v[g].w * v[g].w;
         }
     }
     ss = block_sum<256>(ss, scratch);
@@ -158,7 +173,7 @@ __global__ __launch_bounds__(256) void rmsnorm_wide_kernel(float* __restrict__ x
 #pragma unroll
     for (int g = 0; g < G; ++g) {
         if (threadIdx.x + g * 256 >= ng) continue;
-        const f32x4 o = v[g] * wv[g] * inv;
+        const f32x4 o = v[g] * wv[g] * inv + bv[g];
         typedef OutT out4_t __attribute__((ext_vector_type(4)));  // the group's four values in one store
         const out4_t o4 = {from_f32<OutT>(o.x), from_f32<OutT>(o.y), from_f32<OutT>(o.z), from_f32<OutT>(o.w)};
         *reinterpret_cast<out4_t*>(dst + (size_t)at[g] * 4) = o4;
@@ -404,22 +419,20 @@ extern "C" int ms_feed_tokens(int* tokens, const int* sampled, const int* rows, 
 // rows may be null (identity).  out is float when out_f32 != 0, else the element type.
 // partials [n_partials, T, d] are pending sums of the stream x [T, d] (n_partials may be 0); see the
 // kernel for what is written back.
-extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T, const int* rows, const float* w,
-                          void* out, int out_f32, int n, int d, float eps, hipStream_t stream) {
-    MS_REQUIRE(n > 0 && d > 0, "rmsnorm: empty problem n=%d d=%d", n, d);
-    MS_REQUIRE(d <= MAX_ROW_FLOATS, "rmsnorm: width %d exceeds the row buffer of %d", d, MAX_ROW_FLOATS);
-    MS_REQUIRE(n_partials == 0 || partials, "rmsnorm: %d partial sums without a buffer", n_partials);
-    const size_t ps = (size_t)T * d, smem = (size_t)d * sizeof(float);
-    const bool f32_out = out_f32 || !kHalf;
+// The launch of the kernel above for the widths and numbers of pending sums it is built for; false: not taken.
+template <bool CENTER>
+static bool launch_wide_norm(float* x, const float* partials, int n_partials, size_t ps, const int* rows, const float* w,
+                             const float* bias, void* out, bool f32_out, int n, int d, float eps, hipStream_t stream) {
     const int groups = d % 4 == 0 ? (d <= 1024 ? 1 : (d <= 2048 ? 2 : (d <= 4096 ? 4 : 0))) : 0;
-    const bool aligned = (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(partials)) % 16 == 0;
-    if (groups && aligned && n_partials <= 16) {
-#define MS_NORM(OUT_, G_, NP_)                                                                                   \
-    hipLaunchKernelGGL((rmsnorm_wide_kernel<OUT_, G_, NP_>), dim3(n), dim3(256), 0, stream, x, partials, ps, rows, w, \
-                       (OUT_*)out, d, eps, 0)
-#define MS_NORM_MORE(OUT_, G_)                                                                                          \
-    hipLaunchKernelGGL((rmsnorm_wide_kernel<OUT_, G_, 8, true>), dim3(n), dim3(256), 0, stream, x, partials, ps, rows, w, \
-                       (OUT_*)out, d, eps, n_partials - 8)
+    const bool aligned = (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(partials) |
+                          reinterpret_cast<uintptr_t>(bias)) % 16 == 0;
+    if (!(groups && aligned && n_partials <= 16)) return false;
+#define MS_NORM(OUT_, G_, NP_)                                                                                                      \
+    hipLaunchKernelGGL((rmsnorm_wide_kernel<OUT_, G_, NP_, false, CENTER>), dim3(n), dim3(256), 0, stream, x, partials, ps, rows, w, \
+                       (OUT_*)out, d, eps, 0, bias)
+#define MS_NORM_MORE(OUT_, G_)                                                                                                    \
+    hipLaunchKernelGGL((rmsnorm_wide_kernel<OUT_, G_, 8, true, CENTER>), dim3(n), dim3(256), 0, stream, x, partials, ps, rows, w, \
+                       (OUT_*)out, d, eps, n_partials - 8, bias)
 #define MS_NORM_NP(OUT_, G_)                                    \
     switch (n_partials) {                                       \
         case 0: MS_NORM(OUT_, G_, 0); break;                    \
@@ -437,13 +450,22 @@ extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T
     if (groups == 1) { MS_NORM_NP(OUT_, 1) }                    \
     else if (groups == 2) { MS_NORM_NP(OUT_, 2) }               \
     else { MS_NORM_NP(OUT_, 4) }
-        if (f32_out) { MS_NORM_G(float) } else { MS_NORM_G(elem_t) }
+    if (f32_out) { MS_NORM_G(float) } else { MS_NORM_G(elem_t) }
 #undef MS_NORM_G
 #undef MS_NORM_NP
 #undef MS_NORM_MORE
 #undef MS_NORM
-        return check_launch("rmsnorm");
-    }
+    return true;
+}
+
+extern "C" int ms_rmsnorm(float* x, const float* partials, int n_partials, int T, const int* rows, const float* w,
+                          void* out, int out_f32, int n, int d, float eps, hipStream_t stream) {
+    MS_REQUIRE(n > 0 && d > 0, "rmsnorm: empty problem n=%d d=%d", n, d);
+    MS_REQUIRE(d <= MAX_ROW_FLOATS, "rmsnorm: width %d exceeds the row buffer of %d", d, MAX_ROW_FLOATS);
+    MS_REQUIRE(n_partials == 0 || partials, "rmsnorm: %d partial sums without a buffer", n_partials);
+    const size_t ps = (size_t)T * d, smem = (size_t)d * sizeof(float);
+    const bool f32_out = out_f32 || !kHalf;
+    if (launch_wide_norm<false>(x, partials, n_partials, ps, rows, w, nullptr, out, f32_out, n, d, eps, stream)) return check_launch("rmsnorm");
     if (f32_out)
         hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(n), dim3(256), smem, stream, x, partials, n_partials, ps, rows, w,
                            (float*)out, d, eps);
@@ -459,6 +481,7 @@ extern "C" int ms_layernorm(float* x, const float* partials, int n_partials, int
     MS_REQUIRE(d <= MAX_ROW_FLOATS, "layernorm: width %d exceeds the row buffer of %d", d, MAX_ROW_FLOATS);
     MS_REQUIRE(n_partials == 0 || partials, "layernorm: %d partial sums without a buffer", n_partials);
     const size_t ps = (size_t)T * d, smem = (size_t)d * sizeof(float);
+    if (launch_wide_norm<true>(x, partials, n_partials, ps, rows, w, b, out, out_f32 || !kHalf, n, d, eps, stream)) return check_launch("layernorm");
     if (out_f32 || !kHalf)
         hipLaunchKernelGGL(layernorm_kernel<float>, dim3(n), dim3(256), smem, stream, x, partials, n_partials, ps, rows, w, b,
                            (float*)out, d, eps);

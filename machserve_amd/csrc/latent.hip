@@ -46,12 +46,23 @@ __global__ __launch_bounds__(256) void latent_row_kernel(LatentRowArgs a) {
     const bool kv = a.c_norm != nullptr;
     const int n = a.q_rank + (kv ? a.rank + a.rot : 0);
     float ssq = 0.f, ssc = 0.f;
-    for (int c = threadIdx.x; c < n; c += 256) {
-        float v = 0.f;
-        for (int p = 0; p < a.n_partials; ++p) v += a.proj[p * a.partial_stride + (size_t)t * a.stride + c];
-        row[c] = v;
-        if (c < a.q_rank) ssq += v * v;
-        else if (c < a.q_rank + a.rank) ssc += v * v;
+    // four columns a thread at a time, so that the loads of several columns and partial sums are in flight together
+    for (int c0 = threadIdx.x; c0 < n; c0 += 1024) {
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+        for (int p = 0; p < a.n_partials; ++p) {
+            const float* src = a.proj + p * a.partial_stride + (size_t)t * a.stride;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] += src[min(c0 + u * 256, n - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = c0 + u * 256;
+            if (c >= n) break;
+            row[c] = v[u];
+            if (c < a.q_rank) ssq += v[u] * v[u];
+            else if (c < a.q_rank + a.rank) ssc += v[u] * v[u];
+        }
     }
     ssq = block_sum<256>(ssq, scratch);
     ssc = block_sum<256>(ssc, scratch);
@@ -118,10 +129,8 @@ __global__ __launch_bounds__(256) void latent_query_kernel(const float* __restri
 
 // A product per head: out[t, b, n] = sum_k a[t, b, k] * w[b, n, k], with the rows of `a` and `out` strided (a head's
 // part of a wider row), so that the result lands where its reader wants it.  Operands come straight from memory as
-// fragments (a weight of one head is small and stays in the caches); a wave takes 16 rows by 64 columns.  With
-// ROWS_SPLIT the four waves of a block take 64 rows of one column tile (steps of many rows), otherwise four column
-// tiles of one row tile (decoding).  K is a multiple of 8; what lies beyond it, or beyond the last row or column, is
-// read as zero.
+// fragments (a weight of one head is small and stays in the caches).  K is a multiple of 8; what lies beyond it, or
+// beyond the last row or column, is read as zero.
 struct HeadsLinearArgs {
     const elem_t* a;
     const elem_t* w;  // [B, N, K]
@@ -131,41 +140,54 @@ struct HeadsLinearArgs {
     long ldo, o_head;  // the same in `out`
 };
 
-template <bool ROWS_SPLIT>
+// RT row tiles and CT column tiles of 16 a wave.  WAVES_OVER_ROWS: the block's four waves lie along the rows (a block is
+// 64 * RT rows by 16 * CT columns), else along the columns (16 * RT rows by 64 * CT columns).
+template <int RT, int CT, bool WAVES_OVER_ROWS>
 __global__ __launch_bounds__(256) void heads_linear_kernel(HeadsLinearArgs g) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, grp = lane >> 4;
     const int b = blockIdx.z;
-    const int row0 = ROWS_SPLIT ? blockIdx.x * 64 + wave * 16 : blockIdx.x * 16;
-    const int col0 = ROWS_SPLIT ? blockIdx.y * 64 : (blockIdx.y * 4 + wave) * 64;
+    const int row0 = (WAVES_OVER_ROWS ? blockIdx.x * 4 + wave : blockIdx.x) * 16 * RT;
+    const int col0 = (WAVES_OVER_ROWS ? blockIdx.y : blockIdx.y * 4 + wave) * 16 * CT;
     if (row0 >= g.T || col0 >= g.N) return;  // the same for the whole wave; there is no barrier below
-    const int row = row0 + r16;
-    const elem_t* arow = g.a + (size_t)min(row, g.T - 1) * g.lda + (size_t)b * g.a_head;
+    const elem_t* ab = g.a + (size_t)b * g.a_head;
     const elem_t* wb = g.w + (size_t)b * g.N * g.K;
-    f32x4 acc[4];
+    f32x4 acc[RT][CT];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < RT; ++i)
+#pragma unroll
+        for (int j = 0; j < CT; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < g.K; k0 += 32) {
         const int k = k0 + grp * 8;
         const bool k_in = k < g.K;
-        Frag af = (k_in && row < g.T) ? frag_load(arow + k) : frag_zero();
+        Frag af[RT], bf[CT];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int i = 0; i < RT; ++i) {
+            const int row = row0 + i * 16 + r16;
+            af[i] = (k_in && row < g.T) ? frag_load(ab + (size_t)row * g.lda + k) : frag_zero();
+        }
+#pragma unroll
+        for (int j = 0; j < CT; ++j) {
             const int col = col0 + j * 16 + r16;
-            Frag bf = (k_in && col < g.N) ? frag_load(wb + (size_t)col * g.K + k) : frag_zero();
-            mma_16x16x32(acc[j], af, bf);
+            bf[j] = (k_in && col < g.N) ? frag_load(wb + (size_t)col * g.K + k) : frag_zero();
         }
+#pragma unroll
+        for (int i = 0; i < RT; ++i)
+#pragma unroll
+            for (int j = 0; j < CT; ++j) mma_16x16x32(acc[i][j], af[i], bf[j]);
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int col = col0 + j * 16 + r16;
-        if (col >= g.N) continue;
+    for (int i = 0; i < RT; ++i)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = row0 + grp * 4 + i;
-            if (r < g.T) g.out[(size_t)r * g.ldo + (size_t)b * g.o_head + col] = from_f32<elem_t>(acc[j][i]);
+        for (int j = 0; j < CT; ++j) {
+            const int col = col0 + j * 16 + r16;
+            if (col >= g.N) continue;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int r = row0 + i * 16 + grp * 4 + e;
+                if (r < g.T) g.out[(size_t)r * g.ldo + (size_t)b * g.o_head + col] = from_f32<elem_t>(acc[i][j][e]);
+            }
         }
-    }
 }
 
 }  // namespace ms
@@ -209,10 +231,12 @@ extern "C" int ms_heads_linear(const void* a, long lda, long a_head, const void*
     MS_REQUIRE(B <= 65535, "heads_linear: %d heads", B);
     MS_REQUIRE((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(w)) % 16 == 0, "heads_linear: operands must be 16-byte aligned");
     HeadsLinearArgs g{(const elem_t*)a, (const elem_t*)w, (elem_t*)out, T, B, N, K, lda, a_head, ldo, o_head};
-    if (T > 16) {
-        hipLaunchKernelGGL(heads_linear_kernel<true>, dim3(ceil_div(T, 64), ceil_div(N, 64), B), dim3(256), 0, stream, g);
-    } else {
-        hipLaunchKernelGGL(heads_linear_kernel<false>, dim3(1, ceil_div(N, 256), B), dim3(256), 0, stream, g);
+    if (T >= 256) {  // a wave 64 rows by 64 columns: a weight fragment feeds four products
+        hipLaunchKernelGGL((heads_linear_kernel<4, 4, true>), dim3(ceil_div(T, 256), ceil_div(N, 64), B), dim3(256), 0, stream, g);
+    } else if (T > 16) {
+        hipLaunchKernelGGL((heads_linear_kernel<1, 4, true>), dim3(ceil_div(T, 64), ceil_div(N, 64), B), dim3(256), 0, stream, g);
+    } else {        // few rows: a wave one tile of 16 columns, so that the heads' weights are spread over many waves
+        hipLaunchKernelGGL((heads_linear_kernel<1, 1, false>), dim3(1, ceil_div(N, 64), B), dim3(256), 0, stream, g);
     }
     return check_launch("heads_linear");
 }

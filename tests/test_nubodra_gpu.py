@@ -120,13 +120,13 @@ def test_rotation_of_the_latent_kernels_is_the_plain_models():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,KV,d,taps,temp", [(4, 2, 24, 4, (0.7, 5)), (6, 1, 20, 5, (1.5, 7)), (3, 3, 16, 2, (0.2, 1)), (2, 2, 8, 0, None), (2, 2, 8, 1, None),
-                                              (18, 1, 16, 3, (0.5, 16)), (2, 1, 72, 7, (0.3, 128))])
-def test_rows_behind_the_convolution_in_one_step_and_in_many(dtype, H, KV, d, taps, temp):
+                                              (18, 1, 16, 3, (0.5, 16)), (2, 1, 72, 7, (0.3, 128)), (2, 1, 24, 9, (0.3, 4)), (1, 1, 136, 8, None)])
+@pytest.mark.parametrize("lens", [[11, 1, 6], [75, 1, 40]])
+def test_rows_behind_the_convolution_in_one_step_and_in_many(dtype, H, KV, d, taps, temp, lens):
     ops, ref = ops_of(dtype), EmulatedOps(dtype)
     torch.manual_seed(H * d + taps)
-    ps, hd = 16, -(-d // 16) * 16
+    ps, hd = 128, -(-d // 16) * 16  # a page a request
     C = (H + KV) * d
-    lens = [11, 1, 6]
     T = sum(lens)
     proj = torch.randn(2, T, C + -(-H // 8) * 8)
     conv_w = torch.randn(C, taps) * 0.5 if taps else None
@@ -157,7 +157,7 @@ def test_rows_behind_the_convolution_in_one_step_and_in_many(dtype, H, KV, d, ta
         return torch.stack(qs), torch.stack(gates), kp.float().cpu(), vp.float().cpu(), None if state is None else state.float().cpu()
 
     want = run(ref, [100, 100, 100], lambda t: t.clone())
-    for cuts in ([100, 100, 100], [1, 1, 1], [2, 1, 5], [3, 1, 1]):
+    for cuts in ([100, 100, 100], [1, 1, 1], [2, 1, 5], [3, 1, 1], [64, 1, 29]):
         got = run(ops, cuts, lambda t: dev(t))
         for g, w, what in zip(got, want, ("queries", "gates", "keys", "values", "state")):
             if w is not None:
