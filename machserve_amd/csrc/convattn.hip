@@ -59,7 +59,8 @@ __global__ __launch_bounds__(256) void conv_row_kernel(ConvRowArgs a) {
     const float* st = keep > 0 ? a.state + (size_t)a.seq_slot[s] * keep * C : nullptr;
     auto projected = [&](int r, int c) {
         float v = 0.f;
-        for (int p = 0; p < a.n_partials; ++p) v += a.proj[p * a.partial_stride + (size_t)r * a.stride + c];
+#pragma unroll 8
+        for (int p = 0; p < a.n_partials; ++p) v += a.proj[p * a.partial_stride + (size_t)r * a.stride + c];  // eight loads in flight
         return v;
     };
     for (int c = threadIdx.x; c < C; c += 256) {
@@ -124,7 +125,8 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvRowArgs a, int T) {
     const int C = n_heads * a.d;
     auto projected = [&](int r, int c) {
         float v = 0.f;
-        for (int p = 0; p < a.n_partials; ++p) v += a.proj[p * a.partial_stride + (size_t)r * a.stride + c];
+#pragma unroll 8
+        for (int p = 0; p < a.n_partials; ++p) v += a.proj[p * a.partial_stride + (size_t)r * a.stride + c];  // eight loads in flight
         return v;
     };
     if (hh == n_heads) {
@@ -137,14 +139,19 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvRowArgs a, int T) {
     }
     const int keep = a.taps - 1;
     // per row of the block: how many rows of its request the step holds before it, and the request's state
-    int before[R];
+    // (where every request of the step has one row, row t is request t, which two loads side by side confirm: no search
+    // with its chain of trips to memory; the row's position and address are asked for here, long before they are used)
+    int before[R], pos[R], slot[R];
     const float* st[R];
 #pragma unroll
     for (int i = 0; i < R; ++i) {
         const int t = min(t0 + i, T - 1);
-        const int s = seq_of_row(t, a.seq_q_start, a.S);
+        int s = min(t, a.S - 1);
+        if (!(a.S == T && a.seq_q_start[s] == t && (s == a.S - 1 || a.seq_q_start[s + 1] > t))) s = seq_of_row(t, a.seq_q_start, a.S);
         before[i] = t - a.seq_q_start[s];
         st[i] = keep > 0 ? a.state + (size_t)a.seq_slot[s] * keep * C : nullptr;
+        pos[i] = a.positions[t];
+        slot[i] = a.slot_map[t];
     }
     float y[FAST_CHUNKS][R];
 #pragma unroll
@@ -190,7 +197,7 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvRowArgs a, int T) {
         const float inv = a.unit_norm ? 1.0f / sqrtf(ss / (float)a.d + a.eps) : 1.0f;
         if (hh < a.H) {
             float temp = 1.0f;
-            if (a.temp_coef != 0.f) temp = 1.0f + a.temp_coef * logf((float)((a.positions[t] + 1) / a.temp_every) + 1.0f);
+            if (a.temp_coef != 0.f) temp = 1.0f + a.temp_coef * logf((float)((pos[i] + 1) / a.temp_every) + 1.0f);
             elem_t* dst = a.q_out + ((size_t)t * a.H + hh) * a.dp;
 #pragma unroll
             for (int ci = 0; ci < FAST_CHUNKS; ++ci) {
@@ -198,9 +205,8 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvRowArgs a, int T) {
                 if (e < a.dp) dst[e] = from_f32<elem_t>(e < a.d ? y[ci][i] * inv * temp : 0.f);
             }
         } else {
-            const int slot = a.slot_map[t];
-            if (slot < 0) continue;
-            const int page = slot / a.ps, off = slot % a.ps, kh = hh - a.H;
+            if (slot[i] < 0) continue;
+            const int page = slot[i] / a.ps, off = slot[i] % a.ps, kh = hh - a.H;
             elem_t* krow = a.kpool + (((size_t)page * a.KV + kh) * a.ps + off) * a.dp;
             elem_t* vcol = a.vpool + ((size_t)page * a.KV + kh) * a.dp * a.ps + off;
 #pragma unroll
@@ -230,6 +236,7 @@ __global__ __launch_bounds__(256) void conv_row_state_kernel(const float* __rest
         const int idx = n - keep + i;  // among the step's rows; negative: an older input
         float u = 0.f;
         if (idx >= 0) {
+#pragma unroll 8
             for (int p = 0; p < n_partials; ++p) u += proj[p * partial_stride + (size_t)(q0 + idx) * stride + c];
         } else {
             u = st[(size_t)(keep + idx) * C + c];

@@ -49,7 +49,7 @@ __global__ __launch_bounds__(256) void latent_row_kernel(LatentRowArgs a) {
     // four columns a thread at a time, so that the loads of several columns and partial sums are in flight together
     for (int c0 = threadIdx.x; c0 < n; c0 += 1024) {
         float v[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+#pragma unroll 8
         for (int p = 0; p < a.n_partials; ++p) {
             const float* src = a.proj + p * a.partial_stride + (size_t)t * a.stride;
 #pragma unroll
