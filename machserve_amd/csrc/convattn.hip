@@ -115,6 +115,70 @@ __global__ __launch_bounds__(256) void conv_row_kernel(ConvRowArgs a) {
 // come from its request's state anyway).  The gate's columns are one more "head".  Same sums in the same order as the
 // kernel above.
 constexpr int FAST_TAPS = 8, FAST_CHUNKS = 4;
+
+// A head of a row that is the first of its request in this step (decoding): every earlier input comes from the state.
+// All loads (eight partial sums at a time, the state's rows, the taps' weights, for every chunk of the head) are asked
+// for on one straight path from clamped addresses and picked afterwards, so the wave waits for memory once instead of
+// once a load (a load under a condition makes every later wait a wait for everything).
+__device__ __forceinline__ void conv_head_first_row(const ConvRowArgs& a, int t, int hh, int lane, int slot_of_state, int pos, int slot) {
+    const int n_heads = a.H + a.KV, C = n_heads * a.d, keep = a.taps - 1;
+    const float* st = keep > 0 ? a.state + (size_t)slot_of_state * keep * C : a.proj;
+    const float* row = a.proj + (size_t)t * a.stride;
+    float y[FAST_CHUNKS];
+    float pr[FAST_CHUNKS][8], sv[FAST_CHUNKS][FAST_TAPS - 1], wv[FAST_CHUNKS][FAST_TAPS];
+#pragma unroll
+    for (int ci = 0; ci < FAST_CHUNKS; ++ci) {
+        const int c = hh * a.d + min(lane + 64 * ci, a.d - 1);
+#pragma unroll
+        for (int p = 0; p < 8; ++p) pr[ci][p] = row[(size_t)min(p, a.n_partials - 1) * a.partial_stride + c];
+#pragma unroll
+        for (int k = 0; k < FAST_TAPS - 1; ++k) sv[ci][k] = st[(size_t)min(k, max(keep - 1, 0)) * C + c];
+#pragma unroll
+        for (int k = 0; k < FAST_TAPS; ++k) wv[ci][k] = a.conv_w ? a.conv_w[(size_t)c * a.taps + min(k, keep)] : 1.0f;
+    }
+#pragma unroll
+    for (int ci = 0; ci < FAST_CHUNKS; ++ci) {
+        const int c = hh * a.d + min(lane + 64 * ci, a.d - 1);
+        float u = 0.f;
+#pragma unroll
+        for (int p = 0; p < 8; ++p) u += p < a.n_partials ? pr[ci][p] : 0.f;
+        for (int p = 8; p < a.n_partials; ++p) u += row[(size_t)p * a.partial_stride + c];
+        float acc = 0.f;
+#pragma unroll
+        for (int k = 0; k < FAST_TAPS - 1; ++k) acc += k < keep ? wv[ci][k] * sv[ci][k] : 0.f;
+#pragma unroll
+        for (int k = 0; k < FAST_TAPS; ++k) acc += k == keep ? wv[ci][k] * u : 0.f;
+        y[ci] = lane + 64 * ci < a.d ? acc : 0.f;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int ci = 0; ci < FAST_CHUNKS; ++ci) ss += y[ci] * y[ci];
+    ss = wave_sum(ss);
+    const float inv = a.unit_norm ? 1.0f / sqrtf(ss / (float)a.d + a.eps) : 1.0f;
+    if (hh < a.H) {
+        float temp = 1.0f;
+        if (a.temp_coef != 0.f) temp = 1.0f + a.temp_coef * logf((float)((pos + 1) / a.temp_every) + 1.0f);
+        elem_t* dst = a.q_out + ((size_t)t * a.H + hh) * a.dp;
+#pragma unroll
+        for (int ci = 0; ci < FAST_CHUNKS; ++ci) {
+            const int e = lane + 64 * ci;
+            if (e < a.dp) dst[e] = from_f32<elem_t>(e < a.d ? y[ci] * inv * temp : 0.f);
+        }
+    } else if (slot >= 0) {
+        const int page = slot / a.ps, off = slot % a.ps, kh = hh - a.H;
+        elem_t* krow = a.kpool + (((size_t)page * a.KV + kh) * a.ps + off) * a.dp;
+        elem_t* vcol = a.vpool + ((size_t)page * a.KV + kh) * a.dp * a.ps + off;
+#pragma unroll
+        for (int ci = 0; ci < FAST_CHUNKS; ++ci) {
+            const int e = lane + 64 * ci;
+            if (e < a.d) {
+                krow[e] = from_f32<elem_t>(y[ci] * inv);
+                if (a.values_are_keys) vcol[(size_t)e * a.ps] = from_f32<elem_t>(y[ci]);
+            }
+        }
+    }
+}
+
 template <int R>
 __global__ __launch_bounds__(256) void conv_head_kernel(ConvRowArgs a, int T) {
     constexpr int W = R + FAST_TAPS - 1;
@@ -138,6 +202,13 @@ __global__ __launch_bounds__(256) void conv_head_kernel(ConvRowArgs a, int T) {
         return;
     }
     const int keep = a.taps - 1;
+    if constexpr (R == 1) {
+        // every request of the step has one row, so row t is request t and its first row in this step
+        if (a.S == T && a.seq_q_start[t0] == t0) {
+            conv_head_first_row(a, t0, hh, lane, a.seq_slot[t0], a.positions[t0], a.slot_map[t0]);
+            return;
+        }
+    }
     // per row of the block: how many rows of its request the step holds before it, and the request's state
     // (where every request of the step has one row, row t is request t, which two loads side by side confirm: no search
     // with its chain of trips to memory; the row's position and address are asked for here, long before they are used)
