@@ -84,7 +84,7 @@ struct AttnArgs {
     int nsplit;
     float* part_o;   // [T, H, nsplit, hd]
     float* part_ml;  // [T, H, nsplit, 2]
-    // [H] or null: a softmax sink per head, a term exp(sink) in the denominator that has no key and no value
+    // [H] or null: a softmax sink per head, an extra term exp(sink) of the denominator, to which no key or value belongs
     // (natural-logarithm units of the scaled scores)
     const float* sinks;
     // [T, H] or null: what the output of (row, head) is multiplied by (a gate), in the same pass as the softmax's division

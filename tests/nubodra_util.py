@@ -49,6 +49,13 @@ CONFIGS = {
         latent(5, 8, 4, 8, 12, 12, 0.6, base=100.0, scaling={"factor": 2.0, "original": 16, "fast": 4.0, "slow": 2.0}, ff=56),
         conv_attention(2, 2, 8, 0.7, conv=1, ff=24),
         latent(4, 4, 6, 6, 9, 26, 0.5, base=500.0, kv_from=1, ff=32)], eps=1e-6, scale=1.0),
+    # heads of 64 numbers in both mixers (the attention kernels' tile of 64 takes work items of another size in the
+    # two-byte types, so these heads run in the next tile), attention first, the temperature far beyond the prompts
+    "sixtyfour": model(128, 128, [
+        conv_attention(4, 4, 64, 0.15, conv=3, q_temp=(0.9, 4096), ff=96),
+        latent(8, 32, 16, 64, 64, 48, 0.25, base=50000.0, scaling={"factor": 8.0, "original": 32, "fast": 16.0, "slow": 2.0}, ff=160),
+        latent(2, 64, 16, 32, 32, 48, 0.2, base=50000.0, scaling={"factor": 8.0, "original": 32, "fast": 16.0, "slow": 2.0}, kv_from=1, ff=64),
+        conv_attention(8, 2, 64, 0.1, conv=2, q_temp=(0.1, 2), ff=64)], eps=1e-6, scale=0.5),
     # more heads than a decode tile holds over one latent, more than a few heads a key/value head
     "heads": model(64, 80, [
         latent(20, 8, 8, 8, 32, 40, 0.5, ff=64),

@@ -82,7 +82,7 @@ def query_temperature(n: int, coef: float, every: int, dtype) -> torch.Tensor:
 
 def causal_softmax(scores: torch.Tensor, sink=None) -> torch.Tensor:
     """``scores [heads, n, n]``: softmax over the keys ``j <= i``; with ``sink [heads]`` the denominator also holds
-    ``exp(sink)``, which has no value."""
+    ``exp(sink)``: weight that goes to nothing."""
     n = scores.shape[-1]
     keep = torch.ones(n, n, dtype=torch.bool).tril()
     s = scores.masked_fill(~keep, float("-inf"))
