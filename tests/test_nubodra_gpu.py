@@ -1,8 +1,6 @@
 """Nubodra on the GPU: every new kernel alone against the CPU stand-in of the same entry point (written from the
 mechanisms' equations) or the plain model's function, and the whole engine (cuts of prompts, decoding, mixed batches with
 pages and slots used again, captured steps, generation) against the plain model."""
-import math
-
 import pytest
 import torch
 
@@ -242,7 +240,7 @@ def test_a_sink_far_above_the_scores_takes_the_weight():
     H, hd, ps = 2, 16, 16
     kpool, vpool = torch.randn(2, 1, ps, hd), torch.ones(2, 1, hd, ps)
     q = torch.randn(1, H * hd)
-    table, zero, one = i32([[1]]), i32([0]), i32([1])
+    table = i32([[1]])
     sink = torch.tensor([40.0, -40.0])
     got = ops.decode_attention(dev(q), dev(kpool), dev(vpool), table, i32([3]), H, 1, hd, ps, None, 0.1, dev(sink), None).cpu()
     assert float(got[0, :hd].abs().max()) < 1e-6 and abs(float(got[0, hd]) - 1.0) < 1e-5
